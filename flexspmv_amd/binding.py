@@ -1,0 +1,219 @@
+"""Load a generated gfx950 library and expose the reference's ``merged_spmv_launch`` on it.
+
+The reference's binding is a generated pybind/torch CUDA translation unit
+(cuda_template/merged_binding_template.cu:10-80).  Here the generated library has a C interface
+(``include/flexspmv.h``) and this module is the thin host side above it: it performs the
+reference's argument checks (device, contiguity, dtype, ``ne > 0``; raised as ``RuntimeError`` like
+``TORCH_CHECK``), allocates outputs and scratch with torch's caching allocator, and launches on
+torch's current stream.  Differences from the reference, on purpose:
+
+* outputs are ``torch.empty`` - the kernels write every element exactly once, so the reference's
+  ``torch::zeros`` fill (codegen/merged_gen_binding.py:100-104) is unnecessary traffic;
+* scratch is a cached tensor per (library, device) instead of ``cudaMalloc`` / ``cudaFree`` per
+  call (cuda_template/merged_binding_template.cu:42-49);
+* an unsupported dtype raises (the reference's CUDA binding only logs and falls off the function,
+  :65-68; its CPU binding raises, cpu_template/merged_binding_template_cpu.cpp:45-46).
+
+torch is used for device memory and streams only; there is no CPU or eager fallback: without a
+built library, or without a GPU, calls fail.
+"""
+from __future__ import annotations
+
+import ctypes
+import json
+import os
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+from . import build as _build
+from .ir import FusedGraphIR
+
+ABI_VERSION = 1
+DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
+EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
+                    "flexspmv_last_error", "flexspmv_abi_version")
+
+
+class LaunchArgs(ctypes.Structure):
+    """``flexspmv_launch_args`` of include/flexspmv.h."""
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32),
+        ("value_inputs", ctypes.POINTER(ctypes.c_void_p)),
+        ("num_value_inputs", ctypes.c_int32),
+        ("index_inputs", ctypes.POINTER(ctypes.c_void_p)),
+        ("num_index_inputs", ctypes.c_int32),
+        ("outputs", ctypes.POINTER(ctypes.c_void_p)),
+        ("num_outputs", ctypes.c_int32),
+        ("row_end_offsets", ctypes.c_void_p),
+        ("num_rows", ctypes.c_int64),
+        ("num_cols", ctypes.c_int64),
+        ("ne", ctypes.c_int64),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+        ("stream", ctypes.c_void_p),
+        ("flags", ctypes.c_uint32),
+    ]
+
+
+def load_library(path: str) -> ctypes.CDLL:
+    """dlopen a generated library and type its five entry points."""
+    if not os.path.exists(path):
+        raise RuntimeError(f"FlexSpmv library {path} is not built (run __graft_entry__.build())")
+    lib = ctypes.CDLL(path, mode=ctypes.RTLD_LOCAL)
+    lib.flexspmv_launch.argtypes = [ctypes.POINTER(LaunchArgs)]
+    lib.flexspmv_launch.restype = ctypes.c_int
+    lib.flexspmv_workspace_bytes.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.c_int64]
+    lib.flexspmv_workspace_bytes.restype = ctypes.c_size_t
+    lib.flexspmv_signature.argtypes = []
+    lib.flexspmv_signature.restype = ctypes.c_char_p
+    lib.flexspmv_last_error.argtypes = []
+    lib.flexspmv_last_error.restype = ctypes.c_char_p
+    lib.flexspmv_abi_version.argtypes = []
+    lib.flexspmv_abi_version.restype = ctypes.c_int
+    if lib.flexspmv_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{path}: built for interface version {lib.flexspmv_abi_version()}, "
+                           f"this package speaks {ABI_VERSION}")
+    return lib
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+class HipExtension:
+    """What ``torch.utils.cpp_extension.load`` returns in the reference: an object with
+    ``merged_spmv_launch(values..., gathers..., index tensors..., row_end_offsets, num_rows, num_cols)``.
+    """
+
+    def __init__(self, lib_path: str) -> None:
+        self.lib_path = lib_path
+        self._lib = load_library(lib_path)
+        self.signature: Dict[str, Any] = json.loads(self._lib.flexspmv_signature().decode())
+        self._value_names: List[str] = list(self.signature["value_inputs"])
+        self._index_names: List[str] = list(self.signature["index_inputs"])
+        self._row_aligned = set(self.signature.get("row_aligned_index_inputs", []))
+        self._outputs = self.signature["outputs"]
+        self._has_reducer = bool(self.signature["has_reducer"])
+        self._dtypes = set(self.signature["dtypes"])
+        self._param_names = [p["name"] for p in self.signature["params"]]
+        self._workspace: Dict[Any, Any] = {}
+
+    # -- helpers -------------------------------------------------------------------------
+    def param_names(self) -> List[str]:
+        return list(self._param_names)
+
+    def _bind(self, args: Sequence[Any], kwargs: Dict[str, Any]) -> Dict[str, Any]:
+        names = self._param_names
+        _check(len(args) <= len(names), f"merged_spmv_launch() takes {len(names)} arguments "
+                                         f"({', '.join(names)}), {len(args)} given")
+        bound = dict(zip(names, args))
+        for k, v in kwargs.items():
+            _check(k in names and k not in bound, f"merged_spmv_launch(): unexpected argument {k!r}")
+            bound[k] = v
+        missing = [n for n in names if n not in bound]
+        _check(not missing, f"merged_spmv_launch(): missing arguments {missing}")
+        return bound
+
+    def workspace_bytes(self, dtype: str, num_rows: int, ne: int) -> int:
+        return int(self._lib.flexspmv_workspace_bytes(DTYPE_CODES[dtype], num_rows, ne))
+
+    def _scratch(self, device, nbytes: int):
+        import torch
+        buf = self._workspace.get(device)
+        if buf is None or buf.numel() < nbytes:
+            buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+            self._workspace[device] = buf
+        return buf
+
+    # -- the call ------------------------------------------------------------------------
+    def merged_spmv_launch(self, *args, **kwargs):
+        import torch
+        b = self._bind(args, kwargs)
+        values = [b[n] for n in self._value_names]
+        indices = [b[n] for n in self._index_names]
+        ro = b["row_end_offsets"]
+        num_rows, num_cols = int(b["num_rows"]), int(b["num_cols"])
+
+        dispatch = b[self.signature["dispatch_tensor"]]
+        _check(dispatch.is_cuda, "CUDA device required")
+        for n in self._value_names + self._index_names + ["row_end_offsets"]:
+            t = b[n]
+            _check(t.is_cuda, f"{n} must be a CUDA tensor")
+            _check(t.is_contiguous(), f"{n} must be contiguous")
+        names = {torch.float32: "float32", torch.float64: "float64", torch.int64: "int64"}
+        dt = names.get(dispatch.dtype)
+        _check(dt is not None and dt in self._dtypes and (dt != "int64" or self.signature["allow_int64"]),
+               "Unsupported dtype for ValueT. Use float32 or float64.")
+        for n, t in zip(self._value_names, values):
+            _check(t.dtype == dispatch.dtype, f"{n} dtype mismatch")
+        for n, t in zip(self._index_names, indices):
+            _check(t.dtype == torch.int32, f"{n} dtype mismatch")
+        _check(ro.dtype == torch.int32, "row_end_offsets dtype mismatch")
+
+        ne = int(indices[0].numel()) if indices else num_cols
+        _check(ne > 0, "selector index must be non-empty")
+        for n, t in zip(self._index_names, indices):
+            _check(t.numel() == ne, f"{n} must have ne = {ne} entries")
+        dims = self.signature["value_dims"]
+        for n, t in zip(self._value_names, values):
+            _check(t.numel() % dims[n] == 0, f"{n}.numel() must be a multiple of its item width {dims[n]}")
+        if self._has_reducer:
+            _check(ro.numel() == num_rows + 1, "row_end_offsets must have length num_rows + 1")
+
+        device = dispatch.device
+        outs = []
+        for o in self._outputs:
+            lead = {"reducer": num_rows, "sum": None, "map": ne}[o["kind"]]
+            if lead is None:
+                shape = (o["dim"],)
+            else:
+                shape = (lead,) if o["dim"] == 1 else (lead, o["dim"])
+            outs.append(torch.empty(shape, dtype=dispatch.dtype, device=device))
+
+        ws_bytes = self.workspace_bytes(dt, num_rows, ne)
+        ws = self._scratch(device, ws_bytes)
+
+        def ptr_array(tensors):
+            arr = (ctypes.c_void_p * max(len(tensors), 1))()
+            for i, t in enumerate(tensors):
+                arr[i] = t.data_ptr()
+            return arr
+
+        v_arr, i_arr, o_arr = ptr_array(values), ptr_array(indices), ptr_array(outs)
+        la = LaunchArgs()
+        la.struct_size = ctypes.sizeof(LaunchArgs)
+        la.dtype = DTYPE_CODES[dt]
+        la.value_inputs = ctypes.cast(v_arr, ctypes.POINTER(ctypes.c_void_p))
+        la.num_value_inputs = len(values)
+        la.index_inputs = ctypes.cast(i_arr, ctypes.POINTER(ctypes.c_void_p))
+        la.num_index_inputs = len(indices)
+        la.outputs = ctypes.cast(o_arr, ctypes.POINTER(ctypes.c_void_p))
+        la.num_outputs = len(outs)
+        la.row_end_offsets = ro.data_ptr()
+        la.num_rows, la.num_cols, la.ne = num_rows, num_cols, ne
+        la.workspace, la.workspace_bytes = ws.data_ptr(), ws.numel()
+        with torch.cuda.device(device):
+            la.stream = torch.cuda.current_stream(device).cuda_stream
+            rc = self._lib.flexspmv_launch(ctypes.byref(la))
+        if rc != 0:
+            raise RuntimeError(f"merged_spmv_launch failed ({rc}): {self._lib.flexspmv_last_error().decode()}")
+        if not outs:
+            return None
+        return tuple(outs)
+
+    __call__ = merged_spmv_launch
+
+
+def load_extension(ir: FusedGraphIR, build_if_missing: bool = True) -> HipExtension:
+    """The library of a sub-graph: the prebuilt one when current, else built now with hipcc."""
+    if _build.is_current(ir):
+        return HipExtension(_build.library_path(ir))
+    if not build_if_missing:
+        raise RuntimeError(f"FlexSpmv library for sub-graph {ir.name!r} is not built")
+    return HipExtension(_build.compile_graph(ir))
+
+
+def load_named(name: str, build_if_missing: bool = True) -> HipExtension:
+    from . import graphs
+    return load_extension(graphs.get(name), build_if_missing=build_if_missing)

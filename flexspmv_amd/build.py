@@ -1,0 +1,127 @@
+"""Generate and compile one gfx950 shared library per fused sub-graph.
+
+The reference writes generated sources into its project root / ``include/`` and JIT-builds them with
+``torch.utils.cpp_extension.load`` from a hard-coded path, copying snapshots around so that parallel
+builds do not overwrite each other (test_full/easier_full.py:281-482).  Here every sub-graph gets its
+own directory keyed by the content hash of its six-list description::
+
+    flexspmv_amd/_generated/<name>-<hash>/<name>.hip
+    flexspmv_amd/_generated/<name>-<hash>/lib<name>.so
+
+so builds are independent, cacheable and parallel.  Libraries are built in-tree with ``hipcc
+--offload-arch=gfx950``; a prebuilt library is used as is when its source text is unchanged.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+from typing import Any, Dict, Iterable, List, Optional, Sequence, Tuple
+
+from .ir import FusedGraphIR
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_ROOT = os.path.dirname(PKG_DIR)
+CSRC_DIR = os.path.join(PKG_DIR, "csrc")
+INCLUDE_DIR = os.path.join(REPO_ROOT, "include")
+GENERATED_DIR = os.path.join(PKG_DIR, "_generated")
+
+OFFLOAD_ARCH = "gfx950"
+HIPCC_FLAGS = [
+    f"--offload-arch={OFFLOAD_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed-FP32 instructions are kept out of every kernel of this package
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+]
+
+
+class BuildError(RuntimeError):
+    pass
+
+
+def hipcc_path() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise BuildError("hipcc not found: a generated FlexSpmv library cannot be built on this machine")
+
+
+def _csrc_digest() -> str:
+    h = hashlib.sha1()
+    for root in (CSRC_DIR, INCLUDE_DIR):
+        for fn in sorted(os.listdir(root)):
+            if fn.endswith((".hpp", ".h")):
+                with open(os.path.join(root, fn), "rb") as f:
+                    h.update(fn.encode())
+                    h.update(f.read())
+    return h.hexdigest()[:12]
+
+
+def graph_dir(ir: FusedGraphIR, out_dir: Optional[str] = None) -> str:
+    return os.path.join(out_dir or GENERATED_DIR, f"{ir.name}-{ir.content_hash()}")
+
+
+def write_generated_source(ir: FusedGraphIR, out_dir: Optional[str] = None,
+                           dtypes: Optional[Sequence[str]] = None,
+                           policy: Optional[Dict[str, int]] = None) -> Tuple[str, Dict[str, Any]]:
+    """Emit ``<name>.hip`` for a sub-graph; returns (path, signature)."""
+    from .codegen.merged_gen_gpu import generate_hip_source
+    src, signature = generate_hip_source(ir, dtypes=dtypes, policy=policy)
+    d = graph_dir(ir, out_dir)
+    os.makedirs(d, exist_ok=True)
+    path = os.path.join(d, f"{ir.name}.hip")
+    old = None
+    if os.path.exists(path):
+        with open(path) as f:
+            old = f.read()
+    if old != src:
+        with open(path, "w") as f:
+            f.write(src)
+    return path, signature
+
+
+def library_path(ir: FusedGraphIR, out_dir: Optional[str] = None) -> str:
+    return os.path.join(graph_dir(ir, out_dir), f"lib{ir.name}.so")
+
+
+def _stamp_path(lib: str) -> str:
+    return lib + ".stamp"
+
+
+def _stamp(src_path: str) -> str:
+    with open(src_path, "rb") as f:
+        return hashlib.sha1(f.read()).hexdigest() + ":" + _csrc_digest() + ":" + " ".join(HIPCC_FLAGS)
+
+
+def is_current(ir: FusedGraphIR, out_dir: Optional[str] = None) -> bool:
+    lib = library_path(ir, out_dir)
+    src = os.path.join(graph_dir(ir, out_dir), f"{ir.name}.hip")
+    if not (os.path.exists(lib) and os.path.exists(src) and os.path.exists(_stamp_path(lib))):
+        return False
+    with open(_stamp_path(lib)) as f:
+        return f.read() == _stamp(src)
+
+
+def compile_graph(ir: FusedGraphIR, out_dir: Optional[str] = None, force: bool = False,
+                  dtypes: Optional[Sequence[str]] = None, policy: Optional[Dict[str, int]] = None,
+                  extra_flags: Sequence[str] = ()) -> str:
+    """Generate + compile; returns the path of the shared library."""
+    src, _ = write_generated_source(ir, out_dir, dtypes=dtypes, policy=policy)
+    lib = library_path(ir, out_dir)
+    if not force and is_current(ir, out_dir):
+        return lib
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, f"-I{CSRC_DIR}", f"-I{INCLUDE_DIR}", src, "-o", lib]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise BuildError(f"hipcc failed for sub-graph {ir.name!r}:\n{' '.join(cmd)}\n{proc.stdout}")
+    with open(_stamp_path(lib), "w") as f:
+        f.write(_stamp(src))
+    return lib
+
+
+def compile_many(graphs: Iterable[FusedGraphIR], jobs: int = 8, force: bool = False) -> List[str]:
+    graphs = list(graphs)
+    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(graphs) or 1))) as pool:
+        return list(pool.map(lambda g: compile_graph(g, force=force), graphs))

@@ -1,0 +1,470 @@
+"""Emit the HIP translation unit (gfx950) for one fused sub-graph.
+
+Counterpart of ``generate_cuda_code_from_graph`` (codegen/merged_gen_gpu.py:17-465).  The reference
+pastes per-op statements into CUB-derived agent templates; here the statements are pasted into a graph
+type ``Graph<ValueT>`` consumed by the hand-written kernels of ``csrc/flex_agent.hpp``:
+
+* selector statements follow the reference's emitters (codegen/merged_gen_gpu.py:157-181,
+  codegen/merged_gen_core.py:91-114): an edge tensor is ``Dim`` contiguous values at ``edge*Dim``, a
+  vertex tensor ``Dim`` contiguous values at ``idx[edge]*Dim``;
+* map statements cover the reference's op set with its operator spelling
+  (codegen/merged_gen_gpu.py:188-298): ``add sub mul pow truediv neg add_ exp norm getitem clone copy_
+  setitem abs sign lt gt where`` (``reducer`` / ``sum`` are routed to the reduction machinery);
+* a kernel may hold reducers AND aggregators (the reference's templates hold one or the other,
+  codegen/merged_gen_gpu.py:394);
+* ops that depend on a ``row_aligned`` selector run in the merge walk, where the row is known; the
+  values they need from the coalesced stage travel through LDS next to the reducer arguments.
+"""
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+from ..ir import FusedGraphIR, arg_name, dtype_name, get_dim_length
+from .merged_gen_binding import BindingPlan, binding_plan, generate_binding_code
+
+VERBOSE_ENV = "EASIER_VERBOSE_CODEGEN"  # same switch as the reference (codegen/merged_gen_gpu.py:140)
+
+# LDS a reducer block may use for the per-edge exchange + row offsets; keeps >= 4 blocks per CU
+# (160 KiB LDS per CU on gfx950).
+LDS_BUDGET_BYTES = 36 * 1024
+BLOCK_THREADS = 256
+
+
+@dataclass
+class Var:
+    name: str
+    kind: str          # 'tensor' | 'scalar'
+    dim: int
+    ctype: str         # C++ type name inside Graph<ValueT>
+    stage: int         # stage that defines it: 1 = coalesced edge stage, 2 = merge-walk stage
+    final_stage: int = 1   # stage holding its last value (an in-place op in the walk raises it)
+
+
+@dataclass
+class KernelPlan:
+    plan: BindingPlan
+    vars: Dict[str, Var]
+    exchange: List[Tuple[str, int, int]]      # (variable, component, slot)
+    row_sources: List[Tuple[str, str, int, int]]  # (selector var, source tensor, dim, first slot)
+    red_slices: List[Tuple[str, int, int]]    # (reducer name, first slot, dim)
+    agg_slices: List[Tuple[str, int, int]]
+    xch_width: int = 0
+    red_width: int = 0
+    agg_width: int = 0
+    row_width: int = 0
+
+
+def _literal(a: Any) -> str:
+    if isinstance(a, bool):
+        return "1" if a else "0"
+    if isinstance(a, int):
+        return str(a)
+    if isinstance(a, float):
+        return repr(a)
+    raise TypeError(f"unsupported literal {a!r}")
+
+
+def analyse(ir: FusedGraphIR) -> KernelPlan:
+    """Variable table, stage split and LDS slot assignment for a sub-graph."""
+    inputs, outputs, selector_register, map_ops, red_ops, agg_ops = ir.six()
+    plan = binding_plan(inputs, outputs, selector_register)
+    has_reducer = bool(red_ops)
+    vars: Dict[str, Var] = {}
+
+    cur_stage: Dict[str, int] = {}   # stage a variable's current value lives in (in-place ops may raise it)
+    for s in selector_register:
+        dim = get_dim_length(s["shape"])
+        stage = 2 if (s.get("row_aligned") and has_reducer and s["selector"] == 1) else 1
+        var = s["name"] if s["selector"] == 1 else s["selector_name"]
+        vars[var] = Var(var, "tensor", dim, f"TensorInput_{s['target']}_T", stage)
+        cur_stage[var] = stage
+
+    # values crossing from stage 1 into stage 2 travel through LDS slots
+    exchange: List[Tuple[str, int, int]] = []
+    slot_of: Dict[Tuple[str, int], int] = {}
+
+    def need(var: str) -> None:
+        v = vars[var]
+        for c in range(v.dim):
+            if (var, c) not in slot_of:
+                slot_of[(var, c)] = len(exchange)
+                exchange.append((var, c, len(exchange)))
+
+    # reducer arguments take the first slots so that a plain SpMV exchanges exactly its products
+    red_arg_names = [arg_name(r["args"][0]) for r in red_ops]
+
+    for op in map_ops:
+        o = op["op"]
+        if o in ("reducer", "sum"):
+            continue
+        args = [arg_name(a) for a in (op["args"] if o not in ("getitem", "setitem") else
+                                      [op["args"][0]] + ([op["args"][2]] if o == "setitem" else []))]
+        used = [a for a in args if isinstance(a, str) and a in vars]
+        stage = max([1] + [cur_stage[a] for a in used]) if has_reducer else 1
+        op["_stage"] = stage
+        if stage == 2:
+            for a in used:
+                if vars[a].stage == 1:
+                    need(a)
+        if o in ("setitem", "copy_", "add_"):
+            if o in ("setitem", "add_"):
+                cur_stage[args[0]] = max(cur_stage[args[0]], stage)
+            continue
+        dim = get_dim_length(op["shape"])
+        if o == "norm":
+            vars[op["name"]] = Var(op["name"], "scalar", 1, "ValueT", stage)
+        else:
+            vars[op["name"]] = Var(op["name"], "tensor", dim, f"TensorOutput_{op['name']}_T", stage)
+        cur_stage[op["name"]] = stage
+
+    red_slices, agg_slices = [], []
+    off = 0
+    for r in red_ops:
+        a = arg_name(r["args"][0])
+        dim = get_dim_length(r["shape"])
+        red_slices.append((r["name"], off, dim))
+        off += dim
+        if vars[a].stage == 1:
+            need(a)
+    red_width = off
+    off = 0
+    for g in agg_ops:
+        dim = get_dim_length(g["shape"])
+        agg_slices.append((g["name"], off, dim))
+        off += dim
+    agg_width = off
+    for g in agg_ops:
+        a = arg_name(g["args"][0])
+        if has_reducer and cur_stage[a] == 2 and vars[a].stage == 1:
+            need(a)
+    # put reducer-argument slots first (stable order otherwise)
+    order = sorted(range(len(exchange)), key=lambda i: (exchange[i][0] not in red_arg_names, i))
+    exchange = [(exchange[i][0], exchange[i][1], n) for n, i in enumerate(order)]
+    for var in vars:
+        vars[var].final_stage = cur_stage[var]
+
+    row_sources: List[Tuple[str, str, int, int]] = []
+    row_width = 0
+    for s in selector_register:
+        if s["selector"] == 1 and vars[s["name"]].stage == 2 and s.get("row_aligned"):
+            dim = get_dim_length(s["shape"])
+            row_sources.append((s["name"], s["target"], dim, row_width))
+            row_width += dim
+
+    return KernelPlan(plan, vars, exchange, row_sources, red_slices, agg_slices,
+                      xch_width=len(exchange), red_width=red_width, agg_width=agg_width,
+                      row_width=row_width)
+
+
+# ------------------------------------------------------------------------------------------
+# statement emitters
+# ------------------------------------------------------------------------------------------
+def _arg(a: Any) -> str:
+    a = arg_name(a)
+    return a if isinstance(a, str) else _literal(a)
+
+
+def _emit_selector(s: Dict[str, Any], edge: str) -> List[str]:
+    dim = get_dim_length(s["shape"])
+    if s["selector"] == 1:
+        return [f"const OffsetT column_indices_{s['name']} = flex::stream_load(p.{s['selector_name']}_ptr + {edge});",
+                f"TensorInput_{s['target']}_T {s['name']}(p.{s['target']}_ptr + (size_t)column_indices_{s['name']} * {dim});"]
+    name = s["selector_name"]
+    lines = [f"TensorInput_{s['target']}_T {name};"]
+    lines += [f"{name}.values[{i}] = flex::stream_load(p.{s['target']}_ptr + (size_t){edge} * {dim} + {i});"
+              for i in range(dim)]
+    return lines
+
+
+def _store_loop(ptr: str, edge: str, dim: int, src: str, src_dim: int) -> List[str]:
+    return [f"flex::stream_store({ptr} + (size_t){edge} * {dim} + {i}, {src}.values[{i % src_dim}]);"
+            for i in range(dim)]
+
+
+def _emit_map(op: Dict[str, Any], vars: Dict[str, Var], edge: str) -> List[str]:
+    o, name = op["op"], op["name"]
+    a = [_arg(x) for x in op["args"]] if o not in ("getitem", "setitem") else None
+    T = f"TensorOutput_{name}_T"
+    binary = {"add": "+", "sub": "-", "mul": "*", "pow": "^", "truediv": "/", "lt": "<", "gt": ">"}
+    if o in binary:
+        return [f"{T} {name} = {a[0]} {binary[o]} {a[1]};"]
+    if o == "neg":
+        return [f"{T} {name} = -{a[0]};"]
+    if o in ("exp", "abs", "sign"):
+        return [f"{T} {name} = {a[0]}.{o}();"]
+    if o == "norm":
+        return [f"const ValueT {name} = {a[0]}.l2Norm();"]
+    if o == "where":
+        return [f"{T} {name} = flex::_where({a[0]}, {a[1]}, {a[2]});"]
+    if o == "clone":
+        return [f"{T} {name}({a[0]});"]
+    if o == "getitem":
+        var = _arg(op["args"][0])
+        index = op["args"][1][1]
+        return [f"{T} {name}({var}.values[{int(index)}]);"]
+    dim = get_dim_length(op["shape"])
+    if o == "copy_":
+        dst, src = a[0], a[1]
+        return _store_loop(f"p.{dst}_ptr", edge, dim, src, vars[src].dim)
+    if o == "add_":
+        dst = a[0]
+        return [f"{dst} = {dst} + {a[1]};"] + _store_loop(f"p.{dst}_ptr", edge, dim, dst, vars[dst].dim)
+    if o == "setitem":
+        dst, src = _arg(op["args"][0]), _arg(op["args"][2])
+        sd = vars[src].dim
+        lines = _store_loop(f"p.{dst}_ptr", edge, dim, src, sd)
+        lines += [f"{dst}.values[{i}] = {src}.values[{i % sd}];" for i in range(dim)]
+        return lines
+    raise ValueError(f"Operation {o} not supported")
+
+
+def _component(var: Var, c: int) -> str:
+    return var.name if var.kind == "scalar" else f"{var.name}.values[{c}]"
+
+
+def _indent(lines: Sequence[str], n: int = 4) -> str:
+    pad = " " * n
+    return "".join(pad + l + "\n" for l in lines)
+
+
+def _choose_ipt(kp: KernelPlan, value_bytes: int) -> int:
+    """Items per thread so that one block's LDS stays inside LDS_BUDGET_BYTES."""
+    per_item = 4 + value_bytes * (max(kp.xch_width, 1) + kp.row_width)
+    for ipt in (8, 6, 4, 3, 2, 1):
+        if BLOCK_THREADS * ipt * per_item <= LDS_BUDGET_BYTES:
+            return ipt
+    return 1
+
+
+def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None,
+                        policy: Optional[Dict[str, int]] = None) -> Tuple[str, Dict[str, Any]]:
+    """Return (translation unit text, signature dict) for a sub-graph.
+
+    ``dtypes`` lists the value types to instantiate (default float32 + float64, plus int64 when the
+    dispatch input was traced as int64 - the reference's rule, codegen/merged_gen_binding.py:143-157).
+    ``policy`` may override ``block``, ``ipt_f32``, ``ipt_f64``.
+    """
+    inputs, outputs, selector_register, map_ops, red_ops, agg_ops = ir.six()
+    kp = analyse(ir)
+    plan = kp.plan
+    has_reducer = bool(red_ops)
+    if dtypes is None:
+        dtypes = ["float32", "float64"] + (["int64"] if plan.allow_int64 else [])
+    dtypes = [dtype_name(d) for d in dtypes]
+    policy = dict(policy or {})
+    block = int(policy.get("block", BLOCK_THREADS))
+    ipt = {"float32": int(policy.get("ipt_f32", _choose_ipt(kp, 4))),
+           "float64": int(policy.get("ipt_f64", _choose_ipt(kp, 8))),
+           "int64": int(policy.get("ipt_f64", _choose_ipt(kp, 8)))}
+    if not has_reducer:
+        ipt = {k: int(policy.get("ipt_flat", 8)) for k in ipt}
+
+    # ---- Params ---------------------------------------------------------------------------
+    params, fill = [], []
+    for i, n in enumerate(plan.value_inputs):
+        params.append(f"ValueT* __restrict__ {n}_ptr;")
+        fill.append(f"p.{n}_ptr = static_cast<ValueT*>(a->value_inputs[{i}]);")
+    for i, s in enumerate(plan.selector_inputs):
+        params.append(f"const OffsetT* __restrict__ {s}_ptr;")
+        fill.append(f"p.{s}_ptr = a->index_inputs[{i}];")
+    for i, o in enumerate(plan.outputs):
+        params.append(f"ValueT* __restrict__ output_y_{o.name}_ptr;")
+        fill.append(f"p.output_y_{o.name}_ptr = static_cast<ValueT*>(a->outputs[{i}]);")
+
+    # ---- typedefs -------------------------------------------------------------------------
+    typedefs, seen = [], set()
+    for i in inputs:
+        if i["dtype"] != "int" and i["target"] not in seen:
+            typedefs.append(f"typedef flex::Tensor<ValueT, {get_dim_length(i['shape'])}> TensorInput_{i['target']}_T;")
+            seen.add(i["target"])
+    for op in map_ops:
+        if op["op"] not in ("reducer", "sum", "norm", "setitem", "copy_", "add_"):
+            typedefs.append(f"typedef flex::Tensor<ValueT, {get_dim_length(op['shape'])}> TensorOutput_{op['name']}_T;")
+
+    # ---- stage bodies ---------------------------------------------------------------------
+    s1: List[str] = []
+    s2: List[str] = []
+    for s in selector_register:
+        var = s["name"] if s["selector"] == 1 else s["selector_name"]
+        if kp.vars[var].stage == 1:
+            s1.extend(_emit_selector(s, "e"))
+    # rebuild crossing variables and row-aligned selector values at the top of stage 2
+    rebuilt = set()
+    for var, c, slot in kp.exchange:
+        v = kp.vars[var]
+        if var not in rebuilt:
+            s2.append(f"{v.ctype} {var};" if v.kind == "tensor" else f"ValueT {var};")
+            rebuilt.add(var)
+        s2.append(f"{_component(v, c)} = xch.v[{slot}];")
+    for sel, src, dim, first in kp.row_sources:
+        s2.append(f"TensorInput_{src}_T {sel};")
+        s2 += [f"{sel}.values[{i}] = rv.v[{first + i}];" for i in range(dim)]
+
+    map_output_names = {o.name: o for o in plan.outputs if o.kind == "map"}
+    for op in map_ops:
+        o = op["op"]
+        if o in ("reducer", "sum"):
+            continue
+        stage = op.get("_stage", 1) if has_reducer else 1
+        body = s1 if stage == 1 else s2
+        body.extend(_emit_map(op, kp.vars, "e"))
+        if op["name"] in map_output_names:
+            out = map_output_names[op["name"]]
+            v = kp.vars[op["name"]]
+            if v.kind == "scalar":
+                body.append(f"flex::stream_store(p.output_y_{out.name}_ptr + (size_t)e, {v.name});")
+            else:
+                body.extend(_store_loop(f"p.output_y_{out.name}_ptr", "e", out.dim, v.name, v.dim))
+    # a map output may also be a (stage-1) selector / input variable
+    for name, out in map_output_names.items():
+        if not any(op["name"] == name for op in map_ops):
+            v = kp.vars[name]
+            (s1 if v.stage == 1 or not has_reducer else s2).extend(
+                _store_loop(f"p.output_y_{out.name}_ptr", "e", out.dim, v.name, v.dim))
+
+    # reducer arguments
+    for (rname, first, dim), r in zip(kp.red_slices, red_ops):
+        v = kp.vars[arg_name(r["args"][0])]
+        for c in range(dim):
+            s2.append(f"tot.v[{first + c}] += {_component(v, c % v.dim)};")
+    # aggregator arguments
+    for (gname, first, dim), g in zip(kp.agg_slices, agg_ops):
+        v = kp.vars[arg_name(g["args"][0])]
+        body = s1 if (v.final_stage == 1 or not has_reducer) else s2
+        for c in range(dim):
+            body.append(f"agg.v[{first + c}] += {_component(v, c % v.dim)};")
+    # exchange writes close stage 1
+    if has_reducer:
+        for var, c, slot in kp.exchange:
+            s1.append(f"xch.v[{slot}] = {_component(kp.vars[var], c)};")
+
+    load_row, store_row, add_row, store_agg = [], [], [], []
+    for sel, src, dim, first in kp.row_sources:
+        load_row += [f"rv.v[{first + i}] = p.{src}_ptr[(size_t)row * {dim} + {i}];" for i in range(dim)]
+    for (rname, first, dim) in kp.red_slices:
+        for c in range(dim):
+            store_row.append(f"flex::stream_store(p.output_y_{rname}_ptr + (size_t)row * {dim} + {c}, tot.v[{first + c}]);")
+            add_row.append(f"p.output_y_{rname}_ptr[(size_t)row * {dim} + {c}] += tot.v[{first + c}];")
+    for (gname, first, dim) in kp.agg_slices:
+        for c in range(dim):
+            store_agg.append(f"p.output_y_{gname}_ptr[{c}] = total.v[{first + c}];")
+
+    signature = generate_binding_code(None, inputs, outputs, selector_register)
+    signature.update({
+        "graph": ir.name,
+        "hash": ir.content_hash(),
+        "dtypes": list(dtypes),
+        "row_aligned_index_inputs": sorted({s["selector_name"] + "_idx" for s in selector_register
+                                            if s.get("row_aligned") and has_reducer}),
+        "policy": {"block": block, "ipt": {k: ipt[k] for k in dtypes}},
+        "widths": {"exchange": kp.xch_width, "reduce": kp.red_width, "aggregate": kp.agg_width,
+                   "row": kp.row_width},
+    })
+    sig_json = json.dumps(signature, sort_keys=True)
+    sig_literal = json.dumps(sig_json)  # a C string literal
+
+    ctype = {"float32": "float", "float64": "double", "int64": "long"}
+    enum = {"float32": "FLEXSPMV_F32", "float64": "FLEXSPMV_F64", "int64": "FLEXSPMV_I64"}
+    cases_run, cases_ws = [], []
+    for d in dtypes:
+        disp = f"flex::Dispatch<Graph<{ctype[d]}>, {block}, {ipt[d]}, {'true' if has_reducer else 'false'}>"
+        cases_run.append(
+            f"    case {enum[d]}: {{ Graph<{ctype[d]}>::Params p; Graph<{ctype[d]}>::fill(p, a); return {disp}::run(p, a); }}\n")
+        cases_ws.append(f"    case {enum[d]}: return {disp}::workspace_bytes(num_rows, ne);\n")
+
+    src = f"""// Generated by flexspmv_amd.codegen.merged_gen_gpu for sub-graph "{ir.name}" ({ir.content_hash()}).
+// Do not edit: regenerate from the six-list description instead.
+#include "flex_dispatch.hpp"
+
+namespace {{
+
+template <typename ValueT>
+struct Graph {{
+  using Value = ValueT;
+  using OffsetT = int;
+  static constexpr int XCH_WIDTH = {kp.xch_width};
+  static constexpr int RED_WIDTH = {kp.red_width};
+  static constexpr int AGG_WIDTH = {kp.agg_width};
+  static constexpr int ROW_WIDTH = {kp.row_width};
+
+  struct Params {{
+{_indent(params)}  }};
+
+{_indent(typedefs, 2)}
+  static void fill(Params& p, const flexspmv_launch_args* a) {{
+{_indent(fill)}  }}
+
+  // coalesced edge stage
+  template <class X, class A>
+  static FLEX_DEV void stage1(const Params& p, const int e, X& xch, A& agg) {{
+{_indent(s1)}  }}
+
+  // merge-walk stage (row known)
+  template <class X, class R, class T, class A>
+  static FLEX_DEV void stage2(const Params& p, const int e, const int row, const X& xch, const R& rv, T& tot, A& agg) {{
+{_indent(s2)}  }}
+
+  template <class R>
+  static FLEX_DEV void load_row(const Params& p, const int row, R& rv) {{
+{_indent(load_row)}  }}
+  template <class T>
+  static FLEX_DEV void store_row(const Params& p, const int row, const T& tot) {{
+{_indent(store_row)}  }}
+  template <class T>
+  static FLEX_DEV void add_row(const Params& p, const int row, const T& tot) {{
+{_indent(add_row)}  }}
+  template <class A>
+  static FLEX_DEV void store_agg(const Params& p, const A& total) {{
+{_indent(store_agg)}  }}
+}};
+
+const char kSignature[] = {sig_literal};
+
+}}  // namespace
+
+extern "C" {{
+
+int flexspmv_abi_version(void) {{ return FLEXSPMV_ABI_VERSION; }}
+const char* flexspmv_signature(void) {{ return kSignature; }}
+const char* flexspmv_last_error(void) {{ return flex::g_last_error; }}
+
+size_t flexspmv_workspace_bytes(int32_t dtype, int64_t num_rows, int64_t ne) {{
+  switch (dtype) {{
+{''.join(cases_ws)}    default: return 0;
+  }}
+}}
+
+int flexspmv_launch(const flexspmv_launch_args* a) {{
+  flex::g_last_error[0] = 0;
+  const int bad = flex::check_counts(a, {len(plan.value_inputs)}, {len(plan.selector_inputs)}, {len(plan.outputs)});
+  if (bad != FLEXSPMV_OK) return bad;
+  switch (a->dtype) {{
+{''.join(cases_run)}    default: return flex::fail(FLEXSPMV_ERR_BAD_DTYPE, "Unsupported dtype for ValueT: this library was not generated for it");
+  }}
+}}
+
+}}  // extern "C"
+"""
+    if os.getenv(VERBOSE_ENV) in ("1", "", "true", "True"):
+        for line in s1:
+            print("Stage-1 code: ", line)
+        for line in s2:
+            print("Stage-2 code: ", line)
+    # the analysis annotates ops with '_stage'; leave the caller's lists as they were
+    for op in map_ops:
+        op.pop("_stage", None)
+    return src, signature
+
+
+def generate_cuda_code_from_graph(submodule, traced_model, out_dir: Optional[str] = None):
+    """Reference entry-point name kept for drivers: trace a fused fx sub-module and emit its HIP
+    source (codegen/merged_gen_gpu.py:17).  Returns (path of the .hip file, signature)."""
+    from ..trace.graph_trace import trace_graph
+    from ..build import write_generated_source
+    six = trace_graph(submodule, traced_model)
+    name = getattr(submodule, "_flexspmv_name", None) or type(submodule).__name__
+    ir = FusedGraphIR(str(name), *six)
+    return write_generated_source(ir, out_dir=out_dir)

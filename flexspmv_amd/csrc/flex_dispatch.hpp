@@ -1,0 +1,132 @@
+// Host-side dispatch shared by every generated library: sizes the tiling, carves the workspace and
+// launches the kernels of flex_agent.hpp on the caller's stream.
+//
+// Replaces the reference's merged_spmv_dispatch / merged_spmv_launch pair
+// (cuda_template/reducer/merged_spmv_template.cuh:22-182): same responsibilities (tile count from
+// num_rows + num_nonzeros, temp-storage carving, optional search kernel, the +1 shift that turns the
+// CSR row pointer into row END offsets at :169), but one call instead of the size-query-then-run
+// protocol, and the caller owns the scratch so nothing is allocated per launch.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "flex_agent.hpp"
+#include "flexspmv.h"
+
+namespace flex {
+
+inline thread_local char g_last_error[512] = "";
+inline int fail(int code, const char* msg) {
+  snprintf(g_last_error, sizeof(g_last_error), "%s", msg);
+  return code;
+}
+inline int fail_hip(hipError_t e, const char* where) {
+  snprintf(g_last_error, sizeof(g_last_error), "%s: %s", where, hipGetErrorString(e));
+  return (int)e;
+}
+
+constexpr size_t align_up(size_t n, size_t a = 256) { return (n + a - 1) / a * a; }
+constexpr int FLAT_MAX_BLOCKS = 256 * 8;  // 256 CUs x 8 resident blocks is plenty for a streaming loop
+constexpr int FIXUP_BLOCK = 256;
+
+template <class G, int BLOCK, int IPT, bool REDUCER>
+struct Dispatch {
+  using V = typename G::Value;
+  static constexpr int TILE = BLOCK * IPT;
+
+  struct Layout {
+    int num_tiles;
+    int flat_blocks;
+    size_t off_coords, off_carry_row, off_carry_val, off_partials, total;
+  };
+
+  static bool layout(int64_t num_rows, int64_t ne, Layout& l) {
+    const int64_t items = REDUCER ? num_rows + ne : ne;
+    if (items <= 0 || num_rows + ne >= ((int64_t)1 << 31) - TILE) return false;
+    l.num_tiles = (int)((items + TILE - 1) / TILE);
+    l.flat_blocks = l.num_tiles < FLAT_MAX_BLOCKS ? l.num_tiles : FLAT_MAX_BLOCKS;
+    size_t off = 0;
+    l.off_coords = off;
+    if (REDUCER) off += align_up(sizeof(int2) * ((size_t)l.num_tiles + 1));
+    l.off_carry_row = off;
+    if (REDUCER) off += align_up(sizeof(int) * (size_t)l.num_tiles);
+    l.off_carry_val = off;
+    if (REDUCER) off += align_up(sizeof(V) * (size_t)l.num_tiles * (G::RED_WIDTH > 0 ? G::RED_WIDTH : 1));
+    l.off_partials = off;
+    const size_t parts = REDUCER ? (size_t)l.num_tiles : (size_t)l.flat_blocks;
+    if (G::AGG_WIDTH > 0) off += align_up(sizeof(V) * parts * G::AGG_WIDTH);
+    l.total = off;
+    return true;
+  }
+
+  static size_t workspace_bytes(int64_t num_rows, int64_t ne) {
+    Layout l;
+    if (!layout(num_rows, ne, l)) return 0;
+    return l.total;
+  }
+
+  static int run(const typename G::Params& p, const flexspmv_launch_args* a) {
+    Layout l;
+    if (a->ne <= 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "selector index must be non-empty (ne > 0)");
+    if (REDUCER && a->num_rows <= 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "num_rows must be positive");
+    if (!layout(a->num_rows, a->ne, l))
+      return fail(FLEXSPMV_ERR_TOO_LARGE, "num_rows + ne must stay below 2^31 (32-bit offsets)");
+    if (l.total > 0 && (a->workspace == nullptr || a->workspace_bytes < l.total))
+      return fail(FLEXSPMV_ERR_WORKSPACE, "workspace is missing or smaller than flexspmv_workspace_bytes()");
+    if (REDUCER && a->row_end_offsets == nullptr)
+      return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "row_end_offsets is required by a reducer sub-graph");
+
+    hipStream_t stream = (hipStream_t)a->stream;
+    char* ws = (char*)a->workspace;
+    V* partials = (V*)(ws + l.off_partials);
+    const int nnz = (int)a->ne;
+
+    if constexpr (REDUCER) {
+      const int num_rows = (int)a->num_rows;
+      const int* row_end = a->row_end_offsets + 1;  // CSR pointer -> row END offsets
+      int2* coords = (int2*)(ws + l.off_coords);
+      int* carry_row = (int*)(ws + l.off_carry_row);
+      V* carry_val = (V*)(ws + l.off_carry_val);
+
+      const int search_blocks = (l.num_tiles + 1 + 255) / 256;
+      hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(256), 0, stream, l.num_tiles, TILE,
+                         row_end, num_rows, nnz, coords);
+      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid_for_tiles(l.num_tiles)), dim3(BLOCK), 0, stream,
+                         p, row_end, num_rows, nnz, (const int2*)coords, l.num_tiles, carry_row, carry_val, partials);
+      const int carry_blocks = (l.num_tiles + FIXUP_BLOCK - 1) / FIXUP_BLOCK;
+      hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK>), dim3(carry_blocks + (G::AGG_WIDTH > 0 ? 1 : 0)),
+                         dim3(FIXUP_BLOCK), 0, stream, p, l.num_tiles, carry_blocks, (const int*)carry_row,
+                         (const V*)carry_val, (const V*)partials, l.num_tiles);
+    } else {
+      hipLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(l.flat_blocks), dim3(BLOCK), 0, stream, p, nnz,
+                         l.num_tiles, partials);
+      if (G::AGG_WIDTH > 0) {
+        hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p, 0, 0,
+                           (const int*)nullptr, (const V*)nullptr, (const V*)partials, l.flat_blocks);
+      }
+    }
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail_hip(e, "kernel launch failed");
+    return FLEXSPMV_OK;
+  }
+};
+
+inline int check_counts(const flexspmv_launch_args* a, int nv, int ni, int no) {
+  if (a == nullptr) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "args is NULL");
+  if (a->struct_size != sizeof(flexspmv_launch_args))
+    return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "struct_size does not match this library's flexspmv_launch_args");
+  if (a->flags != 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "flags must be 0");
+  if (a->num_value_inputs != nv || a->num_index_inputs != ni || a->num_outputs != no)
+    return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "argument counts do not match flexspmv_signature()");
+  if ((nv > 0 && a->value_inputs == nullptr) || (ni > 0 && a->index_inputs == nullptr) ||
+      (no > 0 && a->outputs == nullptr))
+    return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "a pointer array is NULL");
+  for (int i = 0; i < nv; ++i)
+    if (a->value_inputs[i] == nullptr) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "a value input pointer is NULL");
+  for (int i = 0; i < no; ++i)
+    if (a->outputs[i] == nullptr) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "an output pointer is NULL");
+  return FLEXSPMV_OK;
+}
+
+}  // namespace flex

@@ -1,0 +1,98 @@
+/* C interface of a generated FlexSpmv library for MI355X (gfx950).
+ *
+ * One shared library is generated per fused sub-graph (select -> map -> reduce / aggregate).  Every
+ * such library exports the same five symbols below; nothing in the signatures is a torch type, so
+ * any host (Python ctypes, a torch extension, C++) can bind them.
+ *
+ * What each entry point stands in for in the reference:
+ *   flexspmv_launch           merged::merged_spmv_launch<ValueT, OffsetT>(FlexParams, d_temp, temp_bytes,
+ *                             debug, stream)  (cuda_template/reducer/merged_spmv_template.cuh:146-182,
+ *                             cuda_template/aggregator/merged_spmv_template.cuh) as driven by
+ *                             merged_spmv_launch_typed (cuda_template/merged_binding_template.cu:10-53);
+ *                             the pointer arrays replace the generated FlexParams fields
+ *                             (cuda_template/merged_utils_template.cuh:243-262).
+ *   flexspmv_workspace_bytes  the size-query call of the same function with d_temp_storage == NULL
+ *                             (cuda_template/reducer/merged_spmv_template.cuh:83-87).
+ *   flexspmv_signature        the argument list the reference bakes into the generated binding
+ *                             (codegen/merged_gen_binding.py:27-78,112-134); here it is data.
+ *   flexspmv_last_error       the strings TORCH_CHECK raises (cuda_template/merged_binding_template.cu:40-50).
+ *   flexspmv_abi_version      no counterpart; lets a loader reject a stale library.
+ */
+#ifndef FLEXSPMV_H_
+#define FLEXSPMV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLEXSPMV_ABI_VERSION 1
+
+/* Value types a library may have been generated for (flexspmv_launch_args.dtype). */
+enum flexspmv_dtype { FLEXSPMV_F32 = 0, FLEXSPMV_F64 = 1, FLEXSPMV_I64 = 2 };
+
+/* Return codes.  Positive values are hipError_t codes passed through unchanged. */
+enum flexspmv_status {
+  FLEXSPMV_OK = 0,
+  FLEXSPMV_ERR_BAD_ARGUMENT = -1,  /* NULL pointer, wrong count, size <= 0, struct_size mismatch */
+  FLEXSPMV_ERR_BAD_DTYPE = -2,     /* dtype not compiled into this library */
+  FLEXSPMV_ERR_TOO_LARGE = -3,     /* num_rows + ne does not fit 32-bit offsets */
+  FLEXSPMV_ERR_WORKSPACE = -4      /* workspace missing or smaller than flexspmv_workspace_bytes() */
+};
+
+/* Arguments of one launch.  All pointers are device pointers valid on the current device.
+ *   value_inputs   value tensors in binding order: non-gather inputs (placeholder order), then gather
+ *                  sources (order of first use); row-major [n][Dim], contiguous.  In-place map ops
+ *                  (setitem / copy_ / add_) write through these pointers.
+ *   index_inputs   one int32 array of ne entries per unique selector module, binding order.  An array
+ *                  declared row-aligned in flexspmv_signature() is never dereferenced.
+ *   outputs        one buffer per output in binding order: reducer [num_rows][Dim], aggregator [Dim],
+ *                  map output [ne][Dim].  Every element is overwritten; no zero fill is needed.
+ *   row_end_offsets  int32[num_rows + 1] with a leading 0 (CSR row pointer); ignored (may be NULL) by
+ *                  libraries without a reducer.
+ *   ne             number of edges (non-zeros); must be > 0.
+ *   workspace      scratch of at least flexspmv_workspace_bytes(...) bytes, 256-byte aligned; contents
+ *                  are not preserved between calls.
+ *   stream         hipStream_t to launch on (NULL = default stream).  The call is asynchronous.
+ */
+typedef struct flexspmv_launch_args {
+  uint32_t struct_size; /* sizeof(flexspmv_launch_args) */
+  int32_t dtype;        /* enum flexspmv_dtype */
+  void* const* value_inputs;
+  int32_t num_value_inputs;
+  const int32_t* const* index_inputs;
+  int32_t num_index_inputs;
+  void* const* outputs;
+  int32_t num_outputs;
+  const int32_t* row_end_offsets;
+  int64_t num_rows;
+  int64_t num_cols;
+  int64_t ne;
+  void* workspace;
+  size_t workspace_bytes;
+  void* stream;
+  uint32_t flags; /* reserved, must be 0 */
+} flexspmv_launch_args;
+
+/* Run the fused sub-graph once.  Returns FLEXSPMV_OK, a negative flexspmv_status, or a hipError_t. */
+int flexspmv_launch(const flexspmv_launch_args* args);
+
+/* Scratch bytes flexspmv_launch needs for these sizes (0 is a valid answer). */
+size_t flexspmv_workspace_bytes(int32_t dtype, int64_t num_rows, int64_t ne);
+
+/* JSON text describing the binding: argument names and kinds, value widths, outputs, compiled
+ * dtypes and the tile policy.  The pointer stays valid for the life of the library. */
+const char* flexspmv_signature(void);
+
+/* Message of the last failed call on this thread ("" if none). */
+const char* flexspmv_last_error(void);
+
+/* FLEXSPMV_ABI_VERSION the library was built against. */
+int flexspmv_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLEXSPMV_H_ */

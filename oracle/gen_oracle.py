@@ -1,0 +1,238 @@
+"""TEST INFRASTRUCTURE ONLY -- emit the CPU oracle (C++/OpenMP) of one fused sub-graph.
+
+The oracle restates what the reference's CPU path computes for a sub-graph: the statements its
+emitters paste (codegen/merged_gen_core.py) into its two OpenMP skeletons
+(cpu_template/merged_spmv_template_reducer.h, cpu_template/merged_spmv_template_aggregator.h),
+written against oracle/tensor_ref.hpp and oracle/merge_ref.hpp.  Only tests, the smoke check and the
+benchmark's CPU-baseline leg may use it; the shipped package never imports this directory.
+
+Per function, what is followed and what pins it:
+
+* selector statements  - merged_gen_core.py:91-114.  Pinned by the reference-held generated instance
+  merged_spmv.h:130-133 (edge tensors) through tests/golden/merge_kat.json, and by naive gather loops.
+* map statements       - merged_gen_core.py:146-234 (same operator spelling; the value type's corner
+  cases are pinned bit-for-bit by tests/golden/tensor_kat.json).
+* reducer pass         - merged_spmv_template_reducer.h:92-169 with the slots of
+  merged_gen_core.py:287-347: even split of num_rows + nnz merge items over T threads, two diagonal
+  searches, whole rows summed left to right and ASSIGNED, the thread's open last row kept as a carry,
+  carries added sequentially in thread order.  Pinned by scipy.sparse products, naive per-row loops
+  and Laplacian closed forms (tests/test_oracle_pins.py); T <= 256 as in the reference's carry arrays
+  (merged_gen_core.py:74-77).
+* flat pass            - merged_spmv_template_aggregator.h:92-136 with merged_gen_core.py:239-284:
+  edges split by ceil((num_rows + nnz) / T), per-thread partials added in thread order and ASSIGNED.
+  Pinned by math.fsum and by the map-only instance in tests/golden/merge_kat.json.
+
+A sub-graph holding reducers AND aggregators has no single counterpart in the reference (its
+templates hold one or the other, codegen/merged_gen_cpu.py:87-89): the oracle runs the reducer pass,
+then the flat pass with in-place stores switched off, which is what running the reference's two
+kernels over the same inputs yields.
+"""
+from __future__ import annotations
+
+import os
+import sys
+from typing import Any, Dict, List, Sequence
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+from flexspmv_amd.codegen.merged_gen_binding import binding_plan  # noqa: E402
+from flexspmv_amd.ir import FusedGraphIR, arg_name, get_dim_length  # noqa: E402
+
+
+def _lit(a: Any) -> str:
+    a = arg_name(a)
+    if isinstance(a, str):
+        return a
+    if isinstance(a, bool):
+        return "1" if a else "0"
+    if isinstance(a, (int, float)):
+        return repr(a)
+    raise TypeError(f"unsupported argument {a!r}")
+
+
+def _selector_statements(selector_register) -> List[str]:
+    out = []
+    for s in selector_register:
+        dim = get_dim_length(s["shape"])
+        if s["selector"] == 1:   # gathered vertex tensor                       merged_gen_core.py:98-108
+            out.append(f"const int column_indices_{s['name']} = {s['selector_name']}_ptr[e];")
+            out.append(f"TensorInput_{s['target']}_T {s['name']}({s['target']}_ptr + (long)column_indices_{s['name']} * {dim});")
+        else:                    # tensor streamed by edge id                   merged_gen_core.py:109-114
+            out.append(f"TensorInput_{s['target']}_T {s['selector_name']}({s['target']}_ptr + (long)e * {dim});")
+    return out
+
+
+def _store(ptr: str, dim: int, src: str) -> List[str]:
+    return [f"if (stores) for (int i = 0; i < {dim}; i++) {ptr}[(long)e * {dim} + i] = {src}.values[i];"]
+
+
+def _map_statements(map_ops) -> List[str]:
+    out = []
+    binary = {"add": "+", "sub": "-", "mul": "*", "pow": "^", "truediv": "/", "lt": "<", "gt": ">"}
+    for op in map_ops:
+        o, name = op["op"], op["name"]
+        dim = get_dim_length(op["shape"])
+        T = f"TensorOutput_{name}_T"
+        if o in binary:                                                       # :146-165, :222-227
+            out.append(f"{T} {name} = {_lit(op['args'][0])} {binary[o]} {_lit(op['args'][1])};")
+        elif o == "neg":                                                      # :166-169
+            out.append(f"{T} {name} = -{_lit(op['args'][0])};")
+        elif o in ("exp", "abs", "sign"):                                     # :177-180, :216-221
+            out.append(f"{T} {name} = {_lit(op['args'][0])}.{o}();")
+        elif o == "norm":                                                     # :181-183
+            out.append(f"ValueT {name} = {_lit(op['args'][0])}.l2Norm();")
+        elif o == "where":                                                    # :228-231
+            out.append(f"{T} {name} = _where({_lit(op['args'][0])}, {_lit(op['args'][1])}, {_lit(op['args'][2])});")
+        elif o == "getitem":                                                  # :186-190
+            out.append(f"{T} {name}({_lit(op['args'][0])}.values[{int(op['args'][1][1])}]);")
+        elif o == "clone":                                                    # :191-194
+            out.append(f"{T} {name}({_lit(op['args'][0])});")
+        elif o == "copy_":                                                    # :195-201
+            out += _store(f"{_lit(op['args'][0])}_ptr", dim, _lit(op["args"][1]))
+        elif o == "add_":                                                     # :170-176
+            dst = _lit(op["args"][0])
+            out.append(f"{dst} = {dst} + {_lit(op['args'][1])};")
+            out += _store(f"{dst}_ptr", dim, dst)
+        elif o == "setitem":                                                  # :202-213
+            dst, src = _lit(op["args"][0]), _lit(op["args"][2])
+            out += _store(f"{dst}_ptr", dim, src)
+            out.append(f"for (int i = 0; i < {dim}; i++) {dst}.values[i] = {src}.values[i];")
+        elif o in ("reducer", "sum"):                                         # :184-185, :214-215
+            continue
+        else:
+            raise ValueError(f"Operation {o} not supported")
+    return out
+
+
+def generate_oracle_source(ir: FusedGraphIR) -> str:
+    inputs, outputs, selector_register, map_ops, red_ops, agg_ops = ir.six()
+    plan = binding_plan(inputs, outputs, selector_register)
+
+    unpack = []
+    for i, n in enumerate(plan.value_inputs):
+        unpack.append(f"ValueT* {n}_ptr = static_cast<ValueT*>(vin[{i}]);")
+    for i, s in enumerate(plan.selector_inputs):
+        unpack.append(f"const int* {s}_ptr = iin[{i}];")
+    for i, o in enumerate(plan.outputs):
+        unpack.append(f"ValueT* output_y_{o.name}_ptr = static_cast<ValueT*>(out[{i}]);")
+    unpack = [u + " (void)" + u.split("=")[0].split()[-1] + ";" for u in unpack]
+
+    typedefs, seen = [], set()
+    for i in inputs:                                                   # merged_gen_core.py:55-60
+        if i["dtype"] != "int" and i["target"] not in seen:
+            typedefs.append(f"typedef Tensor<ValueT, {get_dim_length(i['shape'])}> TensorInput_{i['target']}_T;")
+            seen.add(i["target"])
+    for op in map_ops:                                                 # merged_gen_core.py:141-144
+        if op["op"] not in ("reducer", "sum", "norm"):
+            typedefs.append(f"typedef Tensor<ValueT, {get_dim_length(op['shape'])}> TensorOutput_{op['name']}_T;")
+    for o in plan.outputs:                                             # merged_gen_core.py:69-82
+        if o.kind in ("reducer", "sum"):
+            typedefs.append(f"typedef Tensor<ValueT, {o.dim}> TensorOutput_{o.name}_T;")
+
+    body = _selector_statements(selector_register) + _map_statements(map_ops)
+    norm_names = {op["name"] for op in map_ops if op["op"] == "norm"}
+    for o in plan.outputs:                                             # merged_gen_core.py:83-89
+        if o.kind == "map":
+            if o.name in norm_names:
+                body.append(f"if (stores) output_y_{o.name}_ptr[e] = {o.name};")
+            else:
+                body += _store(f"output_y_{o.name}_ptr", o.dim, o.name)
+    body_txt = "\n".join("        " + b for b in body)
+
+    def pad(lines, n):
+        return "\n".join(" " * n + l for l in lines)
+
+    red = [(r["name"], get_dim_length(r["shape"]), _lit(r["args"][0])) for r in red_ops]
+    agg = [(g["name"], get_dim_length(g["shape"]), _lit(g["args"][0])) for g in agg_ops]
+
+    src = f"""// Generated by oracle/gen_oracle.py for sub-graph "{ir.name}" ({ir.content_hash()}).  TEST INFRASTRUCTURE ONLY.
+#include <omp.h>
+#include <vector>
+#include "merge_ref.hpp"
+using namespace oracle;
+
+namespace {{
+"""
+    if red:
+        src += f"""
+// Reducer pass: cpu_template/merged_spmv_template_reducer.h:92-169.
+template <typename ValueT>
+void reducer_pass(int num_threads, const int* row_ptr, void* const* vin, const int* const* iin,
+                  void* const* out, int num_rows, int nnz, const bool stores) {{
+  const int* row_end = row_ptr + 1;                                             // :97
+{pad(unpack, 2)}
+{pad(typedefs, 2)}
+{pad([f'std::vector<int> row_carry_out_{n}(num_threads); std::vector<TensorOutput_{n}_T> value_carry_out_{n}(num_threads);' for n, _, _ in red], 2)}
+#pragma omp parallel for schedule(static) num_threads(num_threads)
+  for (int tid = 0; tid < num_threads; tid++) {{
+    const Span span = reducer_thread_span(tid, num_threads, row_end, num_rows, nnz);   // :101-121
+    int e = span.begin.y;
+    for (int row = span.begin.x; row < span.end.x; ++row) {{                     // whole rows :124-144
+{pad([f'TensorOutput_{n}_T reducer_{n}_running_total;' for n, _, _ in red], 6)}
+      for (; e < row_end[row]; ++e) {{
+{body_txt}
+{pad([f'reducer_{n}_running_total += {a};' for n, _, a in red], 8)}
+      }}
+{pad([f'for (int i = 0; i < {d}; i++) output_y_{n}_ptr[(long)row * {d} + i] = reducer_{n}_running_total.values[i];' for n, d, _ in red], 6)}
+    }}
+{pad([f'TensorOutput_{n}_T {n}_running_total_partial;' for n, _, _ in red], 4)}
+    for (; e < span.end.y; ++e) {{                                               // open last row :147-160
+{body_txt}
+{pad([f'{n}_running_total_partial += {a};' for n, _, a in red], 6)}
+    }}
+{pad([f'row_carry_out_{n}[tid] = span.end.x; value_carry_out_{n}[tid] = {n}_running_total_partial;' for n, _, _ in red], 4)}
+  }}
+{pad([f'reducer_carry_fixup<ValueT, {d}>(num_threads, num_rows, row_carry_out_{n}.data(), value_carry_out_{n}.data(), output_y_{n}_ptr);' for n, d, _ in red], 2)}
+}}
+"""
+    if agg or not red:
+        src += f"""
+// Flat pass (aggregators and map-only): cpu_template/merged_spmv_template_aggregator.h:92-136.
+template <typename ValueT>
+void flat_pass(int num_threads, void* const* vin, const int* const* iin, void* const* out,
+               int num_rows, int nnz, const bool stores) {{
+{pad(unpack, 2)}
+{pad(typedefs, 2)}
+{pad([f'std::vector<TensorOutput_{n}_T> {n}_running_carry_out(num_threads);' for n, _, _ in agg], 2)}
+#pragma omp parallel for schedule(static) num_threads(num_threads)
+  for (int tid = 0; tid < num_threads; tid++) {{
+    int first, last;
+    flat_thread_range(tid, num_threads, num_rows, nnz, first, last);            // :99-111
+    for (int e = first; e < last; ++e) {{
+{body_txt}
+{pad([f'{n}_running_carry_out[tid] += {a};' for n, _, a in agg], 6)}
+    }}
+  }}
+{pad([f'aggregator_fixup<ValueT, {d}>(num_threads, {n}_running_carry_out.data(), output_y_{n}_ptr);' for n, d, _ in agg], 2)}
+}}
+"""
+    calls = []
+    if red:
+        calls.append("reducer_pass<ValueT>(num_threads, row_ptr, vin, iin, out, num_rows, ne, true);")
+        if agg:
+            calls.append("flat_pass<ValueT>(num_threads, vin, iin, out, num_rows, ne, false);")
+    else:
+        calls.append("flat_pass<ValueT>(num_threads, vin, iin, out, num_rows, ne, true);")
+    src += f"""
+template <typename ValueT>
+void run_all(int num_threads, const int* row_ptr, void* const* vin, const int* const* iin,
+             void* const* out, int num_rows, int ne) {{
+{pad(calls, 2)}
+}}
+
+}}  // namespace
+
+// dtype: 0 float, 1 double, 2 long.  Pointer arrays are in binding order.  Returns 0, or -1 for a bad
+// dtype, -2 when num_threads exceeds the reference's 256-entry carry arrays.
+extern "C" int oracle_run(int dtype, int num_threads, void* const* vin, const int* const* iin,
+                          void* const* out, const int* row_ptr, int num_rows, int ne) {{
+  if (num_threads < 1 || num_threads > 256) return -2;
+  switch (dtype) {{
+    case 0: run_all<float>(num_threads, row_ptr, vin, iin, out, num_rows, ne); return 0;
+    case 1: run_all<double>(num_threads, row_ptr, vin, iin, out, num_rows, ne); return 0;
+{"    case 2: run_all<long>(num_threads, row_ptr, vin, iin, out, num_rows, ne); return 0;" if plan.allow_int64 else ""}
+    default: return -1;
+  }}
+}}
+"""
+    return src
