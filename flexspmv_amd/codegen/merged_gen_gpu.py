@@ -167,16 +167,24 @@ def _arg(a: Any) -> str:
     return a if isinstance(a, str) else _literal(a)
 
 
-def _emit_selector(s: Dict[str, Any], edge: str) -> List[str]:
+def _emit_selector(s: Dict[str, Any]) -> Tuple[List[str], List[str], List[str], List[str], List[str]]:
+    """Statements of one stage-1 selector entry, split by memory level:
+    (Fetch members, fetch statements, Gather members, gather statements, stage-1 prologue)."""
     dim = get_dim_length(s["shape"])
+    T = f"TensorInput_{s['target']}_T"
     if s["selector"] == 1:
-        return [f"const OffsetT column_indices_{s['name']} = flex::stream_load(p.{s['selector_name']}_ptr + {edge});",
-                f"TensorInput_{s['target']}_T {s['name']}(p.{s['target']}_ptr + (size_t)column_indices_{s['name']} * {dim});"]
+        name, idx = s["name"], f"column_indices_{s['name']}"
+        return ([f"OffsetT {idx};"],
+                [f"f.{idx} = flex::stream_load(p.{s['selector_name']}_ptr + e);"],
+                [f"{T} {name};"],
+                [f"g.{name} = {T}(p.{s['target']}_ptr + (size_t)f.{idx} * {dim});"],
+                [f"{T} {name} = g.{name};"])
     name = s["selector_name"]
-    lines = [f"TensorInput_{s['target']}_T {name};"]
-    lines += [f"{name}.values[{i}] = flex::stream_load(p.{s['target']}_ptr + (size_t){edge} * {dim} + {i});"
-              for i in range(dim)]
-    return lines
+    return ([f"{T} {name};"],
+            [f"f.{name}.values[{i}] = flex::stream_load(p.{s['target']}_ptr + (size_t)e * {dim} + {i});"
+             for i in range(dim)],
+            [], [],
+            [f"{T} {name} = f.{name};"])
 
 
 def _store_loop(ptr: str, edge: str, dim: int, src: str, src_dim: int) -> List[str]:
@@ -232,8 +240,8 @@ def _indent(lines: Sequence[str], n: int = 4) -> str:
 
 def _choose_ipt(kp: KernelPlan, value_bytes: int) -> int:
     """Items per thread so that one block's LDS stays inside LDS_BUDGET_BYTES."""
-    per_item = 4 + value_bytes * (max(kp.xch_width, 1) + kp.row_width)
-    for ipt in (8, 6, 4, 3, 2, 1):
+    per_item = value_bytes * (max(kp.xch_width, 1) + kp.row_width)
+    for ipt in (8, 4, 2, 1):
         if BLOCK_THREADS * ipt * per_item <= LDS_BUDGET_BYTES:
             return ipt
     return 1
@@ -287,10 +295,19 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
     # ---- stage bodies ---------------------------------------------------------------------
     s1: List[str] = []
     s2: List[str] = []
+    fetch_members: List[str] = []
+    fetch_body: List[str] = []
+    gather_members: List[str] = []
+    gather_body: List[str] = []
     for s in selector_register:
         var = s["name"] if s["selector"] == 1 else s["selector_name"]
         if kp.vars[var].stage == 1:
-            s1.extend(_emit_selector(s, "e"))
+            fm, fs, gm, gs, pro = _emit_selector(s)
+            fetch_members += fm
+            fetch_body += fs
+            gather_members += gm
+            gather_body += gs
+            s1 += pro
     # rebuild crossing variables and row-aligned selector values at the top of stage 2
     rebuilt = set()
     for var, c, slot in kp.exchange:
@@ -397,9 +414,20 @@ struct Graph {{
   static void fill(Params& p, const flexspmv_launch_args* a) {{
 {_indent(fill)}  }}
 
-  // coalesced edge stage
+  // streamed per-edge data (edge tensors and selector indices): first memory level
+  struct Fetch {{
+{_indent(fetch_members)}  }};
+  // gathered vertex data: second memory level, addressed through Fetch
+  struct Gather {{
+{_indent(gather_members)}  }};
+  static FLEX_DEV void fetch(const Params& p, const int e, Fetch& f) {{
+{_indent(fetch_body)}  }}
+  static FLEX_DEV void gather(const Params& p, const Fetch& f, Gather& g) {{
+{_indent(gather_body)}  }}
+
+  // coalesced edge stage: the map on fetched + gathered data
   template <class X, class A>
-  static FLEX_DEV void stage1(const Params& p, const int e, X& xch, A& agg) {{
+  static FLEX_DEV void stage1(const Params& p, const int e, const Fetch& f, const Gather& g, X& xch, A& agg) {{
 {_indent(s1)}  }}
 
   // merge-walk stage (row known)

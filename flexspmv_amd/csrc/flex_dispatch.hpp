@@ -27,8 +27,34 @@ inline int fail_hip(hipError_t e, const char* where) {
 }
 
 constexpr size_t align_up(size_t n, size_t a = 256) { return (n + a - 1) / a * a; }
-constexpr int FLAT_MAX_BLOCKS = 256 * 8;  // 256 CUs x 8 resident blocks is plenty for a streaming loop
 constexpr int FIXUP_BLOCK = 256;
+constexpr int MAX_PERSISTENT_BLOCKS = 8192;  // upper bound used to size the aggregator partials
+
+// Number of blocks that are resident at once on the current device for a kernel (all CUs filled),
+// rounded down to a multiple of the XCD count; queried once per kernel and device.
+struct GridCache {
+  int device = -1;
+  int grid = 0;
+};
+template <typename KernelT>
+inline int resident_grid(KernelT kernel, int block_threads, GridCache& cache) {
+  int& cached_device = cache.device;
+  int& cached_grid = cache.grid;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return NUM_XCD;
+  if (device == cached_device && cached_grid > 0) return cached_grid;
+  int cus = 0, per_cu = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block_threads, 0) != hipSuccess || per_cu <= 0)
+    per_cu = 1;
+  int grid = cus * per_cu;
+  grid = grid / NUM_XCD * NUM_XCD;
+  if (grid < NUM_XCD) grid = NUM_XCD;
+  if (grid > MAX_PERSISTENT_BLOCKS) grid = MAX_PERSISTENT_BLOCKS;
+  cached_device = device;
+  cached_grid = grid;
+  return grid;
+}
 
 template <class G, int BLOCK, int IPT, bool REDUCER>
 struct Dispatch {
@@ -45,7 +71,7 @@ struct Dispatch {
     const int64_t items = REDUCER ? num_rows + ne : ne;
     if (items <= 0 || num_rows + ne >= ((int64_t)1 << 31) - TILE) return false;
     l.num_tiles = (int)((items + TILE - 1) / TILE);
-    l.flat_blocks = l.num_tiles < FLAT_MAX_BLOCKS ? l.num_tiles : FLAT_MAX_BLOCKS;
+    l.flat_blocks = l.num_tiles < MAX_PERSISTENT_BLOCKS ? l.num_tiles : MAX_PERSISTENT_BLOCKS;
     size_t off = 0;
     l.off_coords = off;
     if (REDUCER) off += align_up(sizeof(int2) * ((size_t)l.num_tiles + 1));
@@ -54,7 +80,7 @@ struct Dispatch {
     l.off_carry_val = off;
     if (REDUCER) off += align_up(sizeof(V) * (size_t)l.num_tiles * (G::RED_WIDTH > 0 ? G::RED_WIDTH : 1));
     l.off_partials = off;
-    const size_t parts = REDUCER ? (size_t)l.num_tiles : (size_t)l.flat_blocks;
+    const size_t parts = MAX_PERSISTENT_BLOCKS;
     if (G::AGG_WIDTH > 0) off += align_up(sizeof(V) * parts * G::AGG_WIDTH);
     l.total = off;
     return true;
@@ -67,6 +93,7 @@ struct Dispatch {
   }
 
   static int run(const typename G::Params& p, const flexspmv_launch_args* a) {
+    static thread_local GridCache grid_cache;  // one per kernel instantiation and host thread
     Layout l;
     if (a->ne <= 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "selector index must be non-empty (ne > 0)");
     if (REDUCER && a->num_rows <= 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "num_rows must be positive");
@@ -92,18 +119,23 @@ struct Dispatch {
       const int search_blocks = (l.num_tiles + 1 + 255) / 256;
       hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(256), 0, stream, l.num_tiles, TILE,
                          row_end, num_rows, nnz, coords);
-      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid_for_tiles(l.num_tiles)), dim3(BLOCK), 0, stream,
+      int grid = resident_grid(reduce_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
+      const int needed = (l.num_tiles + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
+      if (grid > needed) grid = needed;
+      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream,
                          p, row_end, num_rows, nnz, (const int2*)coords, l.num_tiles, carry_row, carry_val, partials);
       const int carry_blocks = (l.num_tiles + FIXUP_BLOCK - 1) / FIXUP_BLOCK;
       hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK>), dim3(carry_blocks + (G::AGG_WIDTH > 0 ? 1 : 0)),
                          dim3(FIXUP_BLOCK), 0, stream, p, l.num_tiles, carry_blocks, (const int*)carry_row,
-                         (const V*)carry_val, (const V*)partials, l.num_tiles);
+                         (const V*)carry_val, (const V*)partials, grid);
     } else {
-      hipLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(l.flat_blocks), dim3(BLOCK), 0, stream, p, nnz,
+      int grid = resident_grid(flat_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
+      if (grid > l.num_tiles) grid = l.num_tiles;
+      hipLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream, p, nnz,
                          l.num_tiles, partials);
       if (G::AGG_WIDTH > 0) {
         hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p, 0, 0,
-                           (const int*)nullptr, (const V*)nullptr, (const V*)partials, l.flat_blocks);
+                           (const int*)nullptr, (const V*)nullptr, (const V*)partials, grid);
       }
     }
     const hipError_t e = hipGetLastError();
