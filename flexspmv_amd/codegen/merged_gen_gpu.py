@@ -342,22 +342,31 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
             (s1 if v.stage == 1 or not has_reducer else s2).extend(
                 _store_loop(f"p.output_y_{out.name}_ptr", "e", out.dim, v.name, v.dim))
 
+    agg2_mask = 0
+    stage1_has_agg = False
     # reducer arguments
     for (rname, first, dim), r in zip(kp.red_slices, red_ops):
         v = kp.vars[arg_name(r["args"][0])]
         for c in range(dim):
-            s2.append(f"tot.v[{first + c}] += {_component(v, c % v.dim)};")
+            s2.append(f"tot.v[{first + c}] = {_component(v, c % v.dim)};")
     # aggregator arguments
     for (gname, first, dim), g in zip(kp.agg_slices, agg_ops):
         v = kp.vars[arg_name(g["args"][0])]
-        body = s1 if (v.final_stage == 1 or not has_reducer) else s2
+        in_walk = has_reducer and v.final_stage == 2
         for c in range(dim):
-            body.append(f"agg.v[{first + c}] += {_component(v, c % v.dim)};")
+            if in_walk:
+                s2.append(f"agg.v[{first + c}] = {_component(v, c % v.dim)};")
+                agg2_mask |= 1 << (first + c)
+            else:
+                s1.append(f"agg.v[{first + c}] += {_component(v, c % v.dim)};")
+                stage1_has_agg = True
     # exchange writes close stage 1
     if has_reducer:
         for var, c, slot in kp.exchange:
             s1.append(f"xch.v[{slot}] = {_component(kp.vars[var], c)};")
 
+    stage2_pure = not any("stream_store(" in line for line in s2)
+    stage1_pure = not stage1_has_agg and not any("stream_store(" in line for line in s1)
     load_row, store_row, add_row, store_agg = [], [], [], []
     for sel, src, dim, first in kp.row_sources:
         load_row += [f"rv.v[{first + i}] = p.{src}_ptr[(size_t)row * {dim} + {i}];" for i in range(dim)]
@@ -406,6 +415,12 @@ struct Graph {{
   static constexpr int RED_WIDTH = {kp.red_width};
   static constexpr int AGG_WIDTH = {kp.agg_width};
   static constexpr int ROW_WIDTH = {kp.row_width};
+  // stage 2 has no side effects besides its accumulators, so the walk may run it unconditionally
+  static constexpr bool STAGE2_PURE = {'true' if stage2_pure else 'false'};
+  // likewise stage 1 (no stores, no aggregator fed from the coalesced stage)
+  static constexpr bool STAGE1_PURE = {'true' if stage1_pure else 'false'};
+  // aggregator slots fed from the merge walk (the others are summed in stage 1)
+  static constexpr unsigned AGG2_MASK = {agg2_mask}u;
 
   struct Params {{
 {_indent(params)}  }};
@@ -430,9 +445,10 @@ struct Graph {{
   static FLEX_DEV void stage1(const Params& p, const int e, const Fetch& f, const Gather& g, X& xch, A& agg) {{
 {_indent(s1)}  }}
 
-  // merge-walk stage (row known)
+  // merge-walk stage (row known): what edge e contributes to the reducers (tot) and to the
+  // aggregators fed from the walk (agg); both are assigned, the kernel accumulates
   template <class X, class R, class T, class A>
-  static FLEX_DEV void stage2(const Params& p, const int e, const int row, const X& xch, const R& rv, T& tot, A& agg) {{
+  static FLEX_DEV void contrib(const Params& p, const int e, const int row, const X& xch, const R& rv, T& tot, A& agg) {{
 {_indent(s2)}  }}
 
   template <class R>
