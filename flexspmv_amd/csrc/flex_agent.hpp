@@ -36,29 +36,6 @@ namespace flex {
 
 constexpr int NUM_XCD = 8;
 
-// Optional phase timing for tuning builds: with -DFLEX_PHASE_CLOCKS thread 0 of every block adds the
-// clock ticks it spent in each phase of reduce_kernel to g_phase_ticks.  Compiled out otherwise.
-#ifdef FLEX_PHASE_CLOCKS
-__device__ unsigned long long g_phase_ticks[16];
-#define FLEX_TICK_INIT                      \
-  unsigned long long tick_ = wall_clock64(); \
-  unsigned long long ticks_[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}
-#define FLEX_TICK(slot)                                \
-  do {                                                 \
-    const unsigned long long now_ = wall_clock64();    \
-    ticks_[slot] += now_ - tick_;                      \
-    tick_ = now_;                                      \
-  } while (0)
-#define FLEX_TICK_FLUSH                                                          \
-  do {                                                                           \
-    if (threadIdx.x == 0)                                                        \
-      for (int i_ = 0; i_ < 12; ++i_) atomicAdd(&g_phase_ticks[i_], ticks_[i_]); \
-  } while (0)
-#else
-#define FLEX_TICK(slot) do {} while (0)
-#define FLEX_TICK_INIT do {} while (0)
-#define FLEX_TICK_FLUSH do {} while (0)
-#endif
 
 template <typename V, int N> struct Pack { V v[N > 0 ? N : 1]; };
 
@@ -102,51 +79,49 @@ tile_search_kernel(int num_tiles, int tile_items, const int* __restrict__ row_en
   coords[t] = merge_path_search(diag, row_end, num_rows, nnz);
 }
 
-// How persistent blocks share the tiles: block b runs on XCD b % 8 (workgroups are dealt to the XCDs
-// round-robin), XCD k owns the contiguous tile range [k*per, (k+1)*per), and the blocks of one XCD
-// interleave over that range so that at any time an XCD works on neighbouring tiles.
-struct TileWalk {
-  int tile, end, step;
-};
-__device__ __forceinline__ TileWalk tiles_of_block(int block, int grid, int num_tiles) {
+// Which tile a block works on.  By default tile = block: neighbouring tiles run at the same time on
+// different XCDs, which measured fastest on the stencil and mesh workloads.  The tuning switch
+// FLEX_TUNE_XCD_CHUNKS instead gives each XCD (block % 8) a contiguous range of tiles.
+__device__ __forceinline__ int tile_of_block(int block, int num_tiles) {
+#ifdef FLEX_TUNE_XCD_CHUNKS
   const int per = (num_tiles + NUM_XCD - 1) / NUM_XCD;
-  const int xcd = block % NUM_XCD;
-  const int slots = grid / NUM_XCD;  // grid is a multiple of NUM_XCD
-  TileWalk w;
-#ifdef FLEX_TUNE_ROUND_ROBIN_TILES  // tuning switch: plain grid-stride assignment, no XCD locality
-  w.tile = block;
-  w.end = num_tiles;
-  w.step = grid;
-  (void)per; (void)xcd; (void)slots;
+  return (block % NUM_XCD) * per + block / NUM_XCD;
 #else
-  w.tile = xcd * per + block / NUM_XCD;
-  w.end = min((xcd + 1) * per, num_tiles);
-  w.step = slots;
+  (void)num_tiles;
+  return block;
 #endif
-  return w;
+}
+inline int grid_for_tiles(int num_tiles) {
+#ifdef FLEX_TUNE_XCD_CHUNKS
+  return (num_tiles + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
+#else
+  return num_tiles;
+#endif
 }
 
 // ----------------------------------------------------------------------------------------------
-// Reducer kernel.  Persistent blocks; each iteration consumes one merge tile of BLOCK*IPT merge
-// items (row ends + non-zeros):
-//   A  row-end offsets of the tile's rows become a bitmap over merge positions in LDS
-//      (row i ends at merge position (row_end[i] - y0) + i); row-aligned vertex data is staged in LDS
-//   B  second-level loads (gathers) of the block's NEXT tile are issued from its first-level data
-//   C  first-level loads (edge tensors, index arrays, row ends) of the tile AFTER NEXT are issued;
-//      both stay in flight during everything below (about 100 KB per CU must be in flight to
-//      saturate HBM, and registers are the only store large enough for it)
-//   D  the map runs in coalesced edge order; values needed per row go to LDS
-//   E  one wavefront turns the bitmap into per-word prefix counts
-//   F  each thread owns IPT consecutive merge items: its bitmap bits say which are row ends and a
-//      popcount gives its merge coordinate (the result of the per-thread diagonal search of the
-//      reference, cuda_template/reducer/merged_agent_spmv_template.cuh:196-215, without a search),
-//      so its LDS reads are independent and the walk is branch-free register work; finished rows go
-//      to an LDS output buffer
-//   G  wave64 DPP segmented scan of the threads' open totals and a fold across waves; each thread
-//      adds its carry-in to the first row it closed
-//   H  the tile's rows leave LDS as coalesced stores
-// The kernel is bound by instruction issue as much as by memory, so loads are never placed under a
-// branch (out-of-range lanes read a clamped address) and per-item work is predicated, not branched.
+// Reducer kernel.  One block per merge tile of BLOCK*IPT merge items (R row ends + Z non-zeros,
+// R + Z = BLOCK*IPT), found by the tile search kernel.  Blocks are small and independent; overlap of
+// one block's memory waits with another block's arithmetic is left to the hardware scheduler (7-8
+// resident blocks per CU), which measured far better than a persistent, software-pipelined loop.
+//
+//   1  first-level loads: IPT edges per thread in coalesced order (edge tensors, index arrays), the
+//      end offset of tile row tid (first wavefront: also of row BLOCK + tid) and row-aligned sources
+//   2  second-level loads: gathers through the index arrays
+//   3  the map runs in coalesced edge order; per-edge values needed per row go to LDS
+//   4  a block-wide vote picks the reduction:
+//      ROW path (every row of the tile has at most ROW_PATH_MAX_LEN non-zeros - meshes, stencils):
+//        thread r owns tile row r, sums its products from LDS and stores the result; consecutive
+//        threads write consecutive rows.  Book-keeping is per row, not per item.
+//      MERGE path (skewed rows): each thread owns IPT consecutive merge items as in the reference
+//        (cuda_template/reducer/merged_agent_spmv_template.cuh:196-345).  Row ends become a bitmap
+//        over merge positions in LDS (row i ends at position (row_end[i] - y0) + i); a popcount
+//        replaces the per-thread diagonal search, so all LDS reads are independent and the walk is
+//        branch-free register work; finished rows go through an LDS buffer to coalesced stores; open
+//        totals are combined by a wave64 DPP segmented scan and a fold across waves.
+// Loads are never placed under a branch (that would serialise them behind a wait each): out-of-range
+// lanes read a clamped address, and per-item work is predicated.  Every row is written exactly once;
+// the tile's open last row becomes a carry record for fixup_kernel.
 // ----------------------------------------------------------------------------------------------
 template <class G, int BLOCK, int IPT>
 __global__ void __launch_bounds__(BLOCK)
@@ -159,174 +134,179 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
   constexpr int NWORDS = TILE / 32;
   constexpr int XCH = G::XCH_WIDTH, RED = G::RED_WIDTH, AGG = G::AGG_WIDTH, ROW = G::ROW_WIDTH;
   constexpr int REDN = RED > 0 ? RED : 1;
-  constexpr int OUT_CAP = 2 * BLOCK;        // finished rows of a tile buffered in LDS
+  constexpr int XCHN = XCH > 0 ? XCH : 1;
+  constexpr int OUT_CAP = 2 * BLOCK;          // merge path: finished rows of a tile buffered in LDS
   constexpr int OUT_STRIDE = OUT_CAP + WAVE;  // + one dump slot per lane for items that close no row
+  constexpr int ROW_PATH_MAX_LEN = 32;        // longest row the row path accepts
+  constexpr int ROW_PATH_UNROLL = 8;          // non-zeros of a row read from LDS up front
+  constexpr int ROW_PATH_MAX_ROWS = BLOCK + WAVE;  // rows (incl. the open one) whose ends are prefetched
   static_assert((IPT & (IPT - 1)) == 0 && IPT <= 32, "a thread's items must sit inside one bitmap word");
   static_assert(NWORDS <= WAVE, "one wavefront scans the bitmap words");
 
-  __shared__ V s_xch[(XCH > 0 ? XCH : 1) * TILE];
-  __shared__ V s_row[(ROW > 0 ? ROW * (TILE + 1) : 1)];
+  __shared__ V s_xch[XCHN * TILE];
   __shared__ V s_out[REDN * OUT_STRIDE];
-  __shared__ unsigned s_bits[2][NWORDS];
+  __shared__ int s_rend[ROW_PATH_MAX_ROWS + 1];  // s_rend[i + 1] = end of tile row i relative to the tile's first non-zero
+  __shared__ unsigned s_bits[NWORDS];
   __shared__ int s_word_prefix[NWORDS];
   __shared__ int s_wave_key[NW];
   __shared__ V s_wave_val[NW][REDN];
   __shared__ V s_wave_agg[NW][AGG > 0 ? AGG : 1];
 
+  const int tile = tile_of_block(blockIdx.x, num_tiles);
+  if (tile >= num_tiles) return;
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
 
-  TileWalk tw = tiles_of_block(blockIdx.x, gridDim.x, num_tiles);
-  Pack<V, AGG> agg;
-  zero(agg);
-  if (tid < NWORDS) {
-    s_bits[0][tid] = 0u;
-    s_bits[1][tid] = 0u;
-  }
-  __syncthreads();
-  if (tw.tile >= tw.end) {
-    // a block without tiles still owns an aggregator partial slot
-    if constexpr (AGG > 0) {
-      if (tid == 0) {
-#pragma unroll
-        for (int c = 0; c < AGG; ++c) agg_partials[(size_t)blockIdx.x * AGG + c] = V(0);
-      }
-    }
-    return;
-  }
-
+  const int2 c0 = coords[tile];
+  const int2 c1 = coords[tile + 1];
+  const int x0 = c0.x, y0 = c0.y;
+  const int R = c1.x - c0.x;  // row ends inside this tile
+  const int Z = c1.y - c0.y;  // non-zeros inside this tile
   const int last_edge = nnz - 1;
   const int last_row = num_rows - 1;
 
-  // First-level loads of a tile starting at merge coordinate c: IPT edges per thread in coalesced
-  // order plus one row per thread.  When the whole window is in range (every tile but the last few)
-  // addresses are linear in the thread id; otherwise they are clamped to the last valid element.
-  auto prefetch = [&](const int2 c, typename G::Fetch (&f)[IPT], int& re, Pack<V, ROW>& rowv) {
-    if (c.y + TILE <= nnz && c.x + BLOCK <= num_rows) {
+  // 1: first-level loads.  A tile holds Z <= TILE non-zeros; lanes past Z re-read the tile's last
+  // edge (one cache line, no extra traffic) instead of running into the next tile's edges.
+  typename G::Fetch f[IPT];
+  const int e_last = min(y0 + max(Z - 1, 0), last_edge);
 #pragma unroll
-      for (int k = 0; k < IPT; ++k) G::fetch(p, c.y + tid + k * BLOCK, f[k]);
-      re = row_end[c.x + tid];
-      if constexpr (ROW > 0) G::load_row(p, c.x + tid, rowv);
-    } else {
-#pragma unroll
-      for (int k = 0; k < IPT; ++k) G::fetch(p, min(c.y + tid + k * BLOCK, last_edge), f[k]);
-      re = row_end[min(c.x + tid, last_row)];
-      if constexpr (ROW > 0) G::load_row(p, min(c.x + tid, last_row), rowv);
+  for (int k = 0; k < IPT; ++k) G::fetch(p, min(y0 + tid + k * BLOCK, e_last), f[k]);
+  int re, re2 = 0;
+  Pack<V, ROW> rowv, rowv2;
+  {
+    const int r1 = min(x0 + tid, last_row);
+    re = row_end[r1];
+    if constexpr (ROW > 0) G::load_row(p, r1, rowv);
+    if (wave == 0) {
+      const int r2 = min(x0 + BLOCK + tid, min(x0 + R, last_row));
+      re2 = row_end[r2];
+      if constexpr (ROW > 0) G::load_row(p, r2, rowv2);
     }
-  };
+  }
 
-  // Software pipeline over this block's tiles t(i) = first + i*step, all state in registers:
-  //   fetch(i+2) and gather(i+1) are issued at the top of iteration i and stay in flight while
-  //   tile i is processed from data that was issued one iteration earlier.
-  // Tile ids past the block's range map to the empty tile at the end of the merge path.
-  auto coord_of = [&](int t, int2& lo, int2& hi) {
-    const int u = (t < tw.end) ? t : num_tiles;
-    lo = coords[u];
-    hi = coords[min(u + 1, num_tiles)];
-  };
-  int2 c0, c1, b0, b1, d0c, d1c, e0, e1;
-  coord_of(tw.tile, c0, c1);
-  coord_of(tw.tile + tw.step, b0, b1);
-  coord_of(tw.tile + 2 * tw.step, d0c, d1c);
-
-  typename G::Fetch fa[IPT], fb[IPT];
-  typename G::Gather ga[IPT];
-  int re_a, re_b;
-  Pack<V, ROW> rowv_a, rowv_b;
-  prefetch(c0, fa, re_a, rowv_a);
-  prefetch(b0, fb, re_b, rowv_b);
+  // 2: gathers
+  typename G::Gather g[IPT];
 #pragma unroll
-  for (int k = 0; k < IPT; ++k) G::gather(p, fa[k], ga[k]);
+  for (int k = 0; k < IPT; ++k) G::gather(p, f[k], g[k]);
 
-  int buf = 0;
-  FLEX_TICK_INIT;
-  for (int tile = tw.tile; tile < tw.end; tile += tw.step, buf ^= 1) {
-    const int x0 = c0.x, y0 = c0.y;
-    const int R = c1.x - c0.x;  // row ends inside this tile
-    const int Z = c1.y - c0.y;  // non-zeros inside this tile
-    coord_of(tile + 3 * tw.step, e0, e1);
+  // tile-relative row ends into LDS; entry R, the row still open at the end of the tile, ends
+  // where the tile ends
+  if (tid == 0) s_rend[0] = 0;
+  if (tid <= R) s_rend[tid + 1] = (tid < R) ? re - y0 : Z;
+  if (wave == 0 && BLOCK + tid <= R && BLOCK + tid < ROW_PATH_MAX_ROWS)
+    s_rend[BLOCK + tid + 1] = (BLOCK + tid < R) ? re2 - y0 : Z;
+  if (tid < NWORDS) s_bits[tid] = 0u;
 
-    // B: gathers of the next tile (its first-level data was issued one iteration ago)
-    typename G::Gather gb[IPT];
+  // 3: map in coalesced order.  Without side effects it runs for every lane (slots past Z are never
+  // read back as non-zeros); with stores or stage-1 aggregators it is predicated.
+  Pack<V, AGG> agg;
+  zero(agg);
 #pragma unroll
-    for (int k = 0; k < IPT; ++k) G::gather(p, fb[k], gb[k]);
+  for (int k = 0; k < IPT; ++k) {
+    const int j = k * BLOCK + tid;
+    if (G::STAGE1_PURE || j < Z) {
+      Pack<V, XCH> xv;
+      G::stage1(p, y0 + j, f[k], g[k], xv, agg);
+#pragma unroll
+      for (int c = 0; c < XCH; ++c) s_xch[c * TILE + j] = xv.v[c];
+    }
+  }
+  __syncthreads();
 
-    // C: first-level loads of the tile after next
-    typename G::Fetch fc[IPT];
-    int re_c;
-    Pack<V, ROW> rowv_c;
-    prefetch(d0c, fc, re_c, rowv_c);
-    FLEX_TICK(0);
+  // 4: vote - can every row of this tile be summed by one thread?
+  const bool few_rows = (R + 1 <= ROW_PATH_MAX_ROWS);
+  int start1 = 0, len1 = 0, start2 = 0, len2 = 0;
+  if (few_rows) {
+    if (tid <= R) {
+      start1 = s_rend[tid];
+      len1 = s_rend[tid + 1] - start1;
+    }
+    if (wave == 0 && BLOCK + tid <= R) {
+      start2 = s_rend[BLOCK + tid];
+      len2 = s_rend[BLOCK + tid + 1] - start2;
+    }
+  }
+  const bool irregular = __syncthreads_or((max(len1, len2) > ROW_PATH_MAX_LEN) | !few_rows);
 
-    // A: row ends -> bitmap; row-aligned sources -> LDS (both prefetched for the first BLOCK rows)
+  if (!irregular) {
+    // ---------------- ROW path ----------------
+    auto sum_row = [&](const int r, const int start, const int len, const Pack<V, ROW>& rv) {
+      Pack<V, XCH> xv[ROW_PATH_UNROLL];
+#pragma unroll
+      for (int it = 0; it < ROW_PATH_UNROLL; ++it) {
+        const int yi = min(start + it, TILE - 1);
+#pragma unroll
+        for (int c = 0; c < XCH; ++c) xv[it].v[c] = s_xch[c * TILE + yi];
+      }
+      Pack<V, RED> tot;
+      zero(tot);
+      auto add_edge = [&](const int yi, const Pack<V, XCH>& x) {
+        Pack<V, RED> dt;
+        Pack<V, AGG> da;
+        G::contrib(p, y0 + yi, x0 + r, x, rv, dt, da);
+#pragma unroll
+        for (int c = 0; c < RED; ++c) tot.v[c] += dt.v[c];
+#pragma unroll
+        for (int c = 0; c < AGG; ++c)
+          if ((G::AGG2_MASK >> c) & 1u) agg.v[c] += da.v[c];
+      };
+#pragma unroll
+      for (int it = 0; it < ROW_PATH_UNROLL; ++it) {
+        if (it < len) add_edge(start + it, xv[it]);
+      }
+      for (int it = ROW_PATH_UNROLL; it < len; ++it) {
+        Pack<V, XCH> x;
+#pragma unroll
+        for (int c = 0; c < XCH; ++c) x.v[c] = s_xch[c * TILE + start + it];
+        add_edge(start + it, x);
+      }
+      if (r < R) {
+        G::store_row(p, x0 + r, tot);
+      } else {  // r == R: the row still open at the end of the tile becomes the tile's carry
+        const int row = x0 + r;
+        carry_row[tile] = (row < num_rows) ? row : -1;
+#pragma unroll
+        for (int c = 0; c < RED; ++c) carry_val[(size_t)tile * RED + c] = tot.v[c];
+      }
+    };
+    if (tid <= R) sum_row(tid, start1, len1, rowv);
+    if (wave == 0 && BLOCK + tid <= R) sum_row(BLOCK + tid, start2, len2, rowv2);
+  } else {
+    // ---------------- MERGE path ----------------
+    // row ends -> bitmap over merge positions (rows beyond the prefetched ones are read here)
     if (tid < R) {
-      const int pos = (re_a - y0) + tid;
-      atomicOr(&s_bits[buf][pos >> 5], 1u << (pos & 31));
+      const int pos = (re - y0) + tid;
+      atomicOr(&s_bits[pos >> 5], 1u << (pos & 31));
     }
     for (int i = tid + BLOCK; i < R; i += BLOCK) {
       const int pos = (row_end[x0 + i] - y0) + i;
-      atomicOr(&s_bits[buf][pos >> 5], 1u << (pos & 31));
+      atomicOr(&s_bits[pos >> 5], 1u << (pos & 31));
     }
-    if constexpr (ROW > 0) {
-      if (tid <= R) {
-#pragma unroll
-        for (int c = 0; c < ROW; ++c) s_row[c * (TILE + 1) + tid] = rowv_a.v[c];
-      }
-      for (int i = tid + BLOCK; i <= R; i += BLOCK) {
-        Pack<V, ROW> rv;
-        G::load_row(p, min(x0 + i, last_row), rv);
-#pragma unroll
-        for (int c = 0; c < ROW; ++c) s_row[c * (TILE + 1) + i] = rv.v[c];
-      }
-    }
-    FLEX_TICK(1);
-
-    // D: map in coalesced order.  Without side effects it runs for every lane (slots past Z are
-    // never read back as non-zeros); with stores or stage-1 aggregators it is predicated.
-#pragma unroll
-    for (int k = 0; k < IPT; ++k) {
-      const int j = k * BLOCK + tid;
-      if (G::STAGE1_PURE || j < Z) {
-        Pack<V, XCH> xv;
-        G::stage1(p, y0 + j, fa[k], ga[k], xv, agg);
-#pragma unroll
-        for (int c = 0; c < XCH; ++c) s_xch[c * TILE + j] = xv.v[c];
-      }
-    }
-    FLEX_TICK(2);
-#ifndef FLEX_ABLATE_NO_WALK  // tuning switch: stop after the map (measures the memory side alone)
     __syncthreads();
-    FLEX_TICK(3);
-
-    // E: exclusive prefix of the bitmap's per-word popcounts; clear the other bitmap for the next tile
+    // exclusive prefix of the bitmap's per-word popcounts
     if (wave == 0) {
-      int cnt[1] = {lane < NWORDS ? (int)__popc(s_bits[buf][lane < NWORDS ? lane : 0]) : 0};
+      int cnt[1] = {lane < NWORDS ? (int)__popc(s_bits[lane < NWORDS ? lane : 0]) : 0};
       const int own = cnt[0];
       wave_segmented_inclusive_sum<int, 1>(0, cnt);
-      if (lane < NWORDS) {
-        s_word_prefix[lane] = cnt[0] - own;
-        s_bits[buf ^ 1][lane] = 0u;
-      }
+      if (lane < NWORDS) s_word_prefix[lane] = cnt[0] - own;
     }
     __syncthreads();
-    FLEX_TICK(4);
 
-    // F: this thread's IPT merge items
+    // this thread's IPT merge items
     const int tile_items = R + Z;
     const int d0 = tid * IPT;
     const int n_items = max(0, min(IPT, tile_items - d0));
-    const unsigned word = s_bits[buf][d0 >> 5];
+    const unsigned word = s_bits[d0 >> 5];
     const int sh = d0 & 31;
     constexpr unsigned FULL = (IPT == 32) ? 0xffffffffu : ((1u << IPT) - 1u);
     const unsigned ends = (word >> sh) & FULL;                                        // items that are row ends
     const unsigned nzs = ~ends & (n_items >= IPT ? FULL : ((1u << n_items) - 1u));  // ... that are non-zeros
     const int xs = s_word_prefix[d0 >> 5] + __popc(word & ((1u << sh) - 1u));        // rows before my items
     const int ys = d0 - xs;                                                            // non-zeros before them
-    const bool direct = R > OUT_CAP;  // (rare) more rows than the LDS output buffer holds: store directly
+    const bool direct = R > OUT_CAP;  // more rows than the LDS output buffer holds: store directly
 
     Pack<V, XCH> xv[IPT];
-    Pack<V, ROW> rvs[IPT];
     int xrel[IPT];
 #pragma unroll
     for (int it = 0; it < IPT; ++it) {
@@ -335,10 +315,6 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
       const int yi = ys + it - before;  // < TILE by construction
 #pragma unroll
       for (int c = 0; c < XCH; ++c) xv[it].v[c] = s_xch[c * TILE + yi];
-      if constexpr (ROW > 0) {
-#pragma unroll
-        for (int c = 0; c < ROW; ++c) rvs[it].v[c] = s_row[c * (TILE + 1) + xrel[it]];
-      }
     }
 
     Pack<V, RED> tot;
@@ -350,9 +326,10 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
       const bool end = (ends >> it) & 1u;
       Pack<V, RED> dt;
       Pack<V, AGG> da;
-      if constexpr (G::STAGE2_PURE) {
+      Pack<V, ROW> rv;
+      if constexpr (G::STAGE2_PURE && ROW == 0) {
         // the contribution of a non-zero is computed for every item and masked in
-        G::contrib(p, y0 + ys + it - (xrel[it] - xs), x0 + xrel[it], xv[it], rvs[it], dt, da);
+        G::contrib(p, y0 + ys + it - (xrel[it] - xs), x0 + xrel[it], xv[it], rv, dt, da);
 #pragma unroll
         for (int c = 0; c < RED; ++c) tot.v[c] += nz ? dt.v[c] : V(0);
 #pragma unroll
@@ -360,7 +337,10 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
           if ((G::AGG2_MASK >> c) & 1u) agg.v[c] += nz ? da.v[c] : V(0);
       } else {
         if (nz) {
-          G::contrib(p, y0 + ys + it - (xrel[it] - xs), x0 + xrel[it], xv[it], rvs[it], dt, da);
+          // row-aligned sources are read from memory here: graphs that use them are mesh-like and
+          // take the row path, so this is the uncommon case
+          if constexpr (ROW > 0) G::load_row(p, x0 + xrel[it], rv);
+          G::contrib(p, y0 + ys + it - (xrel[it] - xs), x0 + xrel[it], xv[it], rv, dt, da);
 #pragma unroll
           for (int c = 0; c < RED; ++c) tot.v[c] += dt.v[c];
 #pragma unroll
@@ -380,8 +360,7 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
       for (int c = 0; c < RED; ++c) tot.v[c] = end ? V(0) : tot.v[c];
     }
 
-    FLEX_TICK(5);
-    // G: block-wide segmented scan of the open totals, keyed by the row each thread ended in
+    // block-wide segmented scan of the open totals, keyed by the row each thread ended in
     const int key = xs + __popc(ends);
     V run[REDN];
 #pragma unroll
@@ -396,9 +375,7 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
 #pragma unroll
       for (int c = 0; c < RED; ++c) s_wave_val[wave][c] = run[c];
     }
-    FLEX_TICK(6);
     __syncthreads();
-    FLEX_TICK(7);
 
     int pk = -1;
     V pv[REDN];
@@ -447,11 +424,9 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
 #pragma unroll
       for (int c = 0; c < RED; ++c) carry_val[(size_t)tile * RED + c] = run[c];
     }
-    FLEX_TICK(8);
     __syncthreads();
-    FLEX_TICK(9);
 
-    // H: the tile's finished rows leave LDS as coalesced stores
+    // the tile's finished rows leave LDS as coalesced stores
     if (!direct) {
       for (int i = tid; i < R; i += BLOCK) {
         Pack<V, RED> t;
@@ -460,27 +435,9 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
         G::store_row(p, x0 + i, t);
       }
     }
-
-    FLEX_TICK(10);
-#endif
-    // rotate the pipeline
-    c0 = b0; c1 = b1;
-    b0 = d0c; b1 = d1c;
-    d0c = e0; d1c = e1;
-#pragma unroll
-    for (int k = 0; k < IPT; ++k) {
-      fa[k] = fb[k];
-      ga[k] = gb[k];
-      fb[k] = fc[k];
-    }
-    re_a = re_b;
-    rowv_a = rowv_b;
-    re_b = re_c;
-    rowv_b = rowv_c;
   }
 
-  FLEX_TICK_FLUSH;
-  // one aggregator partial per block
+  // one aggregator partial per tile
   if constexpr (AGG > 0) {
     wave_sum_to_last_lane<V, AGG>(agg.v);
     if (lane == WAVE - 1) {
@@ -493,7 +450,7 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
       for (int c = 0; c < AGG; ++c) {
         V s = s_wave_agg[0][c];
         for (int w = 1; w < NW; ++w) s += s_wave_agg[w][c];
-        agg_partials[(size_t)blockIdx.x * AGG + c] = s;
+        agg_partials[(size_t)tile * AGG + c] = s;
       }
     }
   }
@@ -553,42 +510,75 @@ flat_kernel(const typename G::Params p, const int nnz, const int num_tiles,
 }
 
 // ----------------------------------------------------------------------------------------------
-// Fix-up: fold tile carries into their rows (tile order) and finish the aggregators (fixed order).
-// Blocks [0, carry_blocks) handle carries, the last block sums the aggregator partials.
+// Fix-up: fold tile carries into their rows (tile order) and pre-reduce the aggregator partials.
+// Block b handles tiles [b*BLOCK, (b+1)*BLOCK): a thread owns the carry of one tile and, when it is
+// the first tile of a run that carries into the same row, adds the whole run to that row.  The
+// block's aggregator partials are summed in a fixed order into block_partials[b].
 // ----------------------------------------------------------------------------------------------
 template <class G, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
-fixup_kernel(const typename G::Params p, const int num_tiles, const int carry_blocks,
-             const int* __restrict__ carry_row, const typename G::Value* __restrict__ carry_val,
-             const typename G::Value* __restrict__ agg_partials, const int num_partials) {
+fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restrict__ carry_row,
+             const typename G::Value* __restrict__ carry_val, const typename G::Value* __restrict__ agg_partials,
+             typename G::Value* __restrict__ block_partials) {
   using V = typename G::Value;
   constexpr int RED = G::RED_WIDTH, AGG = G::AGG_WIDTH;
   constexpr int NW = BLOCK / WAVE;
-  if ((int)blockIdx.x < carry_blocks) {
-    if constexpr (RED > 0) {
-      const int t = blockIdx.x * BLOCK + threadIdx.x;
-      if (t >= num_tiles) return;
+  const int t = blockIdx.x * BLOCK + threadIdx.x;
+  if constexpr (RED > 0) {
+    if (t < num_tiles) {
       const int row = carry_row[t];
-      if (row < 0) return;
-      if (t > 0 && carry_row[t - 1] == row) return;  // not the first tile of this row's run
-      Pack<V, RED> sum;
+      if (row >= 0 && !(t > 0 && carry_row[t - 1] == row)) {  // first tile of this row's run
+        Pack<V, RED> sum;
 #pragma unroll
-      for (int c = 0; c < RED; ++c) sum.v[c] = carry_val[(size_t)t * RED + c];
-      for (int u = t + 1; u < num_tiles && carry_row[u] == row; ++u) {
+        for (int c = 0; c < RED; ++c) sum.v[c] = carry_val[(size_t)t * RED + c];
+        for (int u = t + 1; u < num_tiles && carry_row[u] == row; ++u) {
 #pragma unroll
-        for (int c = 0; c < RED; ++c) sum.v[c] += carry_val[(size_t)u * RED + c];
+          for (int c = 0; c < RED; ++c) sum.v[c] += carry_val[(size_t)u * RED + c];
+        }
+        G::add_row(p, row, sum);
       }
-      G::add_row(p, row, sum);
     }
-    return;
   }
   if constexpr (AGG > 0) {
     __shared__ V s_wave_agg[NW][AGG];
     Pack<V, AGG> acc;
     zero(acc);
-    for (int j = threadIdx.x; j < num_partials; j += BLOCK) {
+    if (t < num_tiles) {
 #pragma unroll
-      for (int c = 0; c < AGG; ++c) acc.v[c] += agg_partials[(size_t)j * AGG + c];
+      for (int c = 0; c < AGG; ++c) acc.v[c] = agg_partials[(size_t)t * AGG + c];
+    }
+    wave_sum_to_last_lane<V, AGG>(acc.v);
+    if ((threadIdx.x & (WAVE - 1)) == WAVE - 1) {
+#pragma unroll
+      for (int c = 0; c < AGG; ++c) s_wave_agg[threadIdx.x / WAVE][c] = acc.v[c];
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int c = 0; c < AGG; ++c) {
+        V s = s_wave_agg[0][c];
+        for (int w = 1; w < NW; ++w) s += s_wave_agg[w][c];
+        block_partials[(size_t)blockIdx.x * AGG + c] = s;
+      }
+    }
+  }
+}
+
+// Final aggregator sum: one block adds `count` partial vectors in a fixed order and assigns the
+// outputs (the reference assigns too: cpu_template/merged_spmv_template_aggregator.h:75-87).
+template <class G, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+aggregate_kernel(const typename G::Params p, const typename G::Value* __restrict__ partials, const int count) {
+  using V = typename G::Value;
+  constexpr int AGG = G::AGG_WIDTH;
+  constexpr int NW = BLOCK / WAVE;
+  if constexpr (AGG > 0) {
+    __shared__ V s_wave_agg[NW][AGG];
+    Pack<V, AGG> acc;
+    zero(acc);
+    for (int j = threadIdx.x; j < count; j += BLOCK) {
+#pragma unroll
+      for (int c = 0; c < AGG; ++c) acc.v[c] += partials[(size_t)j * AGG + c];
     }
     wave_sum_to_last_lane<V, AGG>(acc.v);
     if ((threadIdx.x & (WAVE - 1)) == WAVE - 1) {

@@ -64,7 +64,8 @@ struct Dispatch {
   struct Layout {
     int num_tiles;
     int flat_blocks;
-    size_t off_coords, off_carry_row, off_carry_val, off_partials, total;
+    int carry_blocks;
+    size_t off_coords, off_carry_row, off_carry_val, off_partials, off_block_partials, total;
   };
 
   static bool layout(int64_t num_rows, int64_t ne, Layout& l) {
@@ -79,9 +80,12 @@ struct Dispatch {
     if (REDUCER) off += align_up(sizeof(int) * (size_t)l.num_tiles);
     l.off_carry_val = off;
     if (REDUCER) off += align_up(sizeof(V) * (size_t)l.num_tiles * (G::RED_WIDTH > 0 ? G::RED_WIDTH : 1));
+    l.carry_blocks = (l.num_tiles + FIXUP_BLOCK - 1) / FIXUP_BLOCK;
     l.off_partials = off;
-    const size_t parts = MAX_PERSISTENT_BLOCKS;
+    const size_t parts = REDUCER ? (size_t)l.num_tiles : (size_t)MAX_PERSISTENT_BLOCKS;
     if (G::AGG_WIDTH > 0) off += align_up(sizeof(V) * parts * G::AGG_WIDTH);
+    l.off_block_partials = off;
+    if (REDUCER && G::AGG_WIDTH > 0) off += align_up(sizeof(V) * (size_t)l.carry_blocks * G::AGG_WIDTH);
     l.total = off;
     return true;
   }
@@ -119,23 +123,23 @@ struct Dispatch {
       const int search_blocks = (l.num_tiles + 1 + 255) / 256;
       hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(256), 0, stream, l.num_tiles, TILE,
                          row_end, num_rows, nnz, coords);
-      int grid = resident_grid(reduce_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
-      const int needed = (l.num_tiles + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
-      if (grid > needed) grid = needed;
-      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream,
+      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid_for_tiles(l.num_tiles)), dim3(BLOCK), 0, stream,
                          p, row_end, num_rows, nnz, (const int2*)coords, l.num_tiles, carry_row, carry_val, partials);
-      const int carry_blocks = (l.num_tiles + FIXUP_BLOCK - 1) / FIXUP_BLOCK;
-      hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK>), dim3(carry_blocks + (G::AGG_WIDTH > 0 ? 1 : 0)),
-                         dim3(FIXUP_BLOCK), 0, stream, p, l.num_tiles, carry_blocks, (const int*)carry_row,
-                         (const V*)carry_val, (const V*)partials, grid);
+      V* block_partials = (V*)(ws + l.off_block_partials);
+      hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0, stream, p,
+                         l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials, block_partials);
+      if (G::AGG_WIDTH > 0) {
+        hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
+                           (const V*)block_partials, l.carry_blocks);
+      }
     } else {
       int grid = resident_grid(flat_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
       if (grid > l.num_tiles) grid = l.num_tiles;
       hipLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream, p, nnz,
                          l.num_tiles, partials);
       if (G::AGG_WIDTH > 0) {
-        hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p, 0, 0,
-                           (const int*)nullptr, (const V*)nullptr, (const V*)partials, grid);
+        hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
+                           (const V*)partials, grid);
       }
     }
     const hipError_t e = hipGetLastError();
