@@ -143,14 +143,16 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
   static_assert((IPT & (IPT - 1)) == 0 && IPT <= 32, "a thread's items must sit inside one bitmap word");
   static_assert(NWORDS <= WAVE, "one wavefront scans the bitmap words");
 
-  __shared__ V s_xch[XCHN * TILE];
-  __shared__ V s_out[REDN * OUT_STRIDE];
-  __shared__ int s_rend[ROW_PATH_MAX_ROWS + 1];  // s_rend[i + 1] = end of tile row i relative to the tile's first non-zero
+  // s_xch holds the per-edge values of the tile; the merge path reuses it (after a barrier) as its
+  // output buffer s_out
+  constexpr int XCH_ELEMS = XCHN * TILE, OUT_ELEMS = REDN * OUT_STRIDE;
+  __shared__ V s_xch[XCH_ELEMS > OUT_ELEMS ? XCH_ELEMS : OUT_ELEMS];
+  V* const s_out = s_xch;
   __shared__ unsigned s_bits[NWORDS];
   __shared__ int s_word_prefix[NWORDS];
+  __shared__ int s_vote[NW];
   __shared__ int s_wave_key[NW];
   __shared__ V s_wave_val[NW][REDN];
-  __shared__ V s_wave_agg[NW][AGG > 0 ? AGG : 1];
 
   const int tile = tile_of_block(blockIdx.x, num_tiles);
   if (tile >= num_tiles) return;
@@ -172,16 +174,21 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
   const int e_last = min(y0 + max(Z - 1, 0), last_edge);
 #pragma unroll
   for (int k = 0; k < IPT; ++k) G::fetch(p, min(y0 + tid + k * BLOCK, e_last), f[k]);
-  int re, re2 = 0;
+  // ... and of the rows: thread tid holds the end of tile row tid, the first wavefront also the end
+  // of row BLOCK + tid; lane 0 of each wavefront fetches the end of the row before its first one,
+  // the other lanes get it from their neighbour, so every thread knows where its row starts.
+  int re, re2 = 0, prev_lane0 = 0, prev2_lane0 = 0;
   Pack<V, ROW> rowv, rowv2;
   {
     const int r1 = min(x0 + tid, last_row);
     re = row_end[r1];
     if constexpr (ROW > 0) G::load_row(p, r1, rowv);
+    if (lane == 0 && tid > 0) prev_lane0 = row_end[min(x0 + tid - 1, last_row)];
     if (wave == 0) {
       const int r2 = min(x0 + BLOCK + tid, min(x0 + R, last_row));
       re2 = row_end[r2];
       if constexpr (ROW > 0) G::load_row(p, r2, rowv2);
+      if (lane == 0) prev2_lane0 = row_end[min(x0 + BLOCK - 1, last_row)];
     }
   }
 
@@ -190,12 +197,6 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
 #pragma unroll
   for (int k = 0; k < IPT; ++k) G::gather(p, f[k], g[k]);
 
-  // tile-relative row ends into LDS; entry R, the row still open at the end of the tile, ends
-  // where the tile ends
-  if (tid == 0) s_rend[0] = 0;
-  if (tid <= R) s_rend[tid + 1] = (tid < R) ? re - y0 : Z;
-  if (wave == 0 && BLOCK + tid <= R && BLOCK + tid < ROW_PATH_MAX_ROWS)
-    s_rend[BLOCK + tid + 1] = (BLOCK + tid < R) ? re2 - y0 : Z;
   if (tid < NWORDS) s_bits[tid] = 0u;
 
   // 3: map in coalesced order.  Without side effects it runs for every lane (slots past Z are never
@@ -212,22 +213,38 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
       for (int c = 0; c < XCH; ++c) s_xch[c * TILE + j] = xv.v[c];
     }
   }
-  __syncthreads();
 
-  // 4: vote - can every row of this tile be summed by one thread?
+  // 4: vote - can every row of this tile be summed by one thread?  Row i of the tile spans the
+  // tile-relative non-zeros [end(i-1), end(i)), with end(-1) = 0 and, for the row still open at the
+  // end of the tile (i == R), end = Z.  The vote doubles as the barrier that publishes s_xch.
   const bool few_rows = (R + 1 <= ROW_PATH_MAX_ROWS);
   int start1 = 0, len1 = 0, start2 = 0, len2 = 0;
-  if (few_rows) {
+  {
+    const int end1 = (tid < R) ? re - y0 : Z;
+    int prev = wave_shift_up1<int>(end1, 0);
+    if (lane == 0) prev = (tid > 0) ? prev_lane0 - y0 : 0;
     if (tid <= R) {
-      start1 = s_rend[tid];
-      len1 = s_rend[tid + 1] - start1;
+      start1 = prev;
+      len1 = end1 - prev;
     }
-    if (wave == 0 && BLOCK + tid <= R) {
-      start2 = s_rend[BLOCK + tid];
-      len2 = s_rend[BLOCK + tid + 1] - start2;
+    if (wave == 0) {
+      const int end2 = (BLOCK + tid < R) ? re2 - y0 : Z;
+      int prev2 = wave_shift_up1<int>(end2, 0);
+      if (lane == 0) prev2 = prev2_lane0 - y0;
+      if (BLOCK + tid <= R) {
+        start2 = prev2;
+        len2 = end2 - prev2;
+      }
     }
   }
-  const bool irregular = __syncthreads_or((max(len1, len2) > ROW_PATH_MAX_LEN) | !few_rows);
+  const bool my_vote = (max(len1, len2) > ROW_PATH_MAX_LEN) | !few_rows;
+  if (lane == 0) s_vote[wave] = (__builtin_amdgcn_ballot_w64(my_vote) != 0ull) ? 1 : 0;
+  else (void)__builtin_amdgcn_ballot_w64(my_vote);
+  __syncthreads();
+  int any_vote = 0;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) any_vote |= s_vote[w];
+  const bool irregular = any_vote != 0;
 
   if (!irregular) {
     // ---------------- ROW path ----------------
@@ -316,6 +333,8 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
 #pragma unroll
       for (int c = 0; c < XCH; ++c) xv[it].v[c] = s_xch[c * TILE + yi];
     }
+
+    __syncthreads();  // every thread has read its s_xch values: the buffer now serves as s_out
 
     Pack<V, RED> tot;
     zero(tot);
@@ -437,21 +456,12 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
     }
   }
 
-  // one aggregator partial per tile
+  // one aggregator partial per wavefront of the tile (fixup_kernel adds them in a fixed order)
   if constexpr (AGG > 0) {
     wave_sum_to_last_lane<V, AGG>(agg.v);
     if (lane == WAVE - 1) {
 #pragma unroll
-      for (int c = 0; c < AGG; ++c) s_wave_agg[wave][c] = agg.v[c];
-    }
-    __syncthreads();
-    if (tid == 0) {
-#pragma unroll
-      for (int c = 0; c < AGG; ++c) {
-        V s = s_wave_agg[0][c];
-        for (int w = 1; w < NW; ++w) s += s_wave_agg[w][c];
-        agg_partials[(size_t)tile * AGG + c] = s;
-      }
+      for (int c = 0; c < AGG; ++c) agg_partials[((size_t)tile * NW + wave) * AGG + c] = agg.v[c];
     }
   }
 }
@@ -513,9 +523,10 @@ flat_kernel(const typename G::Params p, const int nnz, const int num_tiles,
 // Fix-up: fold tile carries into their rows (tile order) and pre-reduce the aggregator partials.
 // Block b handles tiles [b*BLOCK, (b+1)*BLOCK): a thread owns the carry of one tile and, when it is
 // the first tile of a run that carries into the same row, adds the whole run to that row.  The
-// block's aggregator partials are summed in a fixed order into block_partials[b].
+// block's aggregator partials (PARTS_PER_TILE per tile, one per wavefront of the reducer block) are
+// summed in a fixed order into block_partials[b].
 // ----------------------------------------------------------------------------------------------
-template <class G, int BLOCK>
+template <class G, int BLOCK, int PARTS_PER_TILE>
 __global__ void __launch_bounds__(BLOCK)
 fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restrict__ carry_row,
              const typename G::Value* __restrict__ carry_val, const typename G::Value* __restrict__ agg_partials,
@@ -545,7 +556,10 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
     zero(acc);
     if (t < num_tiles) {
 #pragma unroll
-      for (int c = 0; c < AGG; ++c) acc.v[c] = agg_partials[(size_t)t * AGG + c];
+      for (int w = 0; w < PARTS_PER_TILE; ++w) {
+#pragma unroll
+        for (int c = 0; c < AGG; ++c) acc.v[c] += agg_partials[((size_t)t * PARTS_PER_TILE + w) * AGG + c];
+      }
     }
     wave_sum_to_last_lane<V, AGG>(acc.v);
     if ((threadIdx.x & (WAVE - 1)) == WAVE - 1) {

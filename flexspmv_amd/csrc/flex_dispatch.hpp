@@ -82,7 +82,7 @@ struct Dispatch {
     if (REDUCER) off += align_up(sizeof(V) * (size_t)l.num_tiles * (G::RED_WIDTH > 0 ? G::RED_WIDTH : 1));
     l.carry_blocks = (l.num_tiles + FIXUP_BLOCK - 1) / FIXUP_BLOCK;
     l.off_partials = off;
-    const size_t parts = REDUCER ? (size_t)l.num_tiles : (size_t)MAX_PERSISTENT_BLOCKS;
+    const size_t parts = REDUCER ? (size_t)l.num_tiles * (BLOCK / WAVE) : (size_t)MAX_PERSISTENT_BLOCKS;
     if (G::AGG_WIDTH > 0) off += align_up(sizeof(V) * parts * G::AGG_WIDTH);
     l.off_block_partials = off;
     if (REDUCER && G::AGG_WIDTH > 0) off += align_up(sizeof(V) * (size_t)l.carry_blocks * G::AGG_WIDTH);
@@ -126,7 +126,7 @@ struct Dispatch {
       hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid_for_tiles(l.num_tiles)), dim3(BLOCK), 0, stream,
                          p, row_end, num_rows, nnz, (const int2*)coords, l.num_tiles, carry_row, carry_val, partials);
       V* block_partials = (V*)(ws + l.off_block_partials);
-      hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0, stream, p,
+      hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, BLOCK / WAVE>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0, stream, p,
                          l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials, block_partials);
       if (G::AGG_WIDTH > 0) {
         hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
