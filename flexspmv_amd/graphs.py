@@ -193,7 +193,7 @@ def op_zoo(dtype="float32") -> FusedGraphIR:
     b.map("abs", "abs_1", ["sub"])
     b.map("pow", "pow_1", ["abs_1", 0.5])
     b.map("pow", "pow_2", ["abs_1", "c2"], shape=(3,))       # tensor exponent, widths 3 ^ 2
-    b.map("exp", "exp", ["neg"])
+    b.map("exp", "exp", ["sub"])
     b.map("sign", "sign", ["sub"])
     b.map("norm", "norm", ["b3"])
     b.map("truediv", "truediv_2", ["sub", "norm"], shape=(3,))   # tensor / scalar: unguarded
@@ -212,7 +212,9 @@ def op_zoo(dtype="float32") -> FusedGraphIR:
     b.map("setitem", "setitem", ["dst6", (SLICE_ALL,), "add_1"], shape=(6,))
     b.map("add", "add_2", ["where", "where_2"])
     b.map("add", "add_3", ["add_2", "pow_2"])
-    b.map("add", "add_4", ["add_3", "truediv_2"])
+    b.map("mul", "mul_3", ["neg", 0.001])
+    b.map("add", "add_6", ["add_3", "mul_3"])
+    b.map("add", "add_4", ["add_6", "truediv_2"])
     b.map("add", "add_5", ["add_4", "acc"])
     b.reduce("reducer", "add_5")
     b.reduce("reducer_6", "dst6", module="reducer")

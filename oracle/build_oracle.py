@@ -81,6 +81,14 @@ def build_kats() -> Dict[str, str]:
     return out
 
 
+def build_merge_capi() -> str:
+    """C entry points over merge_ref.hpp for the brute-force tests -> oracle/_build/libmerge_ref.so."""
+    os.makedirs(BUILD_DIR, exist_ok=True)
+    lib = os.path.join(BUILD_DIR, "libmerge_ref.so")
+    _run([CXX, "-O2", "-std=c++17", "-fPIC", "-shared", f"-I{HERE}", os.path.join(HERE, "merge_capi.cpp"), "-o", lib])
+    return lib
+
+
 def build_reference_kats(reference_root: str = "/root/reference") -> Dict[str, str]:
     os.makedirs(REF_DIR, exist_ok=True)
     out = {}

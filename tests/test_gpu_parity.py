@@ -1,0 +1,233 @@
+"""Parity of the HIP path with the CPU oracle, through the C interface of the generated libraries
+(ctypes launcher in flexspmv_amd.binding).  Tolerances: float32 1e-5, float64 1e-12, relative to the
+largest magnitude of the output being compared (per-row scale for SpMV); integers and structure exact.
+"""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+
+torch = pytest.importorskip("torch")
+
+from flexspmv_amd import graphs
+from flexspmv_amd import workloads as W
+from flexspmv_amd.binding import load_named
+from oracle.runner import run_oracle
+from tests.util_inputs import STRUCTURES, make_inputs, row_structure
+from tests.test_oracle_pins import op_zoo_inputs
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype("float32"): 1e-5, np.dtype("float64"): 1e-12}
+THREADS = 8   # oracle thread count; its rounding depends on it, which the tolerances absorb
+
+
+def gpu_launch(name, tensors, row_ptr, num_rows, num_cols):
+    """merged_spmv_launch on cuda:0; returns (outputs, value inputs after the call) as numpy."""
+    ext = load_named(name, build_if_missing=False)
+    args, dev_tensors = [], {}
+    for pname in ext.param_names():
+        if pname == "row_end_offsets":
+            ro = row_ptr if row_ptr is not None else np.array([42], dtype=np.int32)
+            args.append(torch.from_numpy(np.ascontiguousarray(ro)).cuda())
+        elif pname == "num_rows":
+            args.append(int(num_rows))
+        elif pname == "num_cols":
+            args.append(int(num_cols))
+        else:
+            dev_tensors[pname] = torch.from_numpy(np.ascontiguousarray(tensors[pname])).cuda()
+            args.append(dev_tensors[pname])
+    outs = ext.merged_spmv_launch(*args)
+    torch.cuda.synchronize()
+    outs = [] if outs is None else [o.cpu().numpy() for o in outs]
+    after = {k: v.cpu().numpy() for k, v in dev_tensors.items() if k in ext.signature["value_inputs"]}
+    return outs, after
+
+
+def assert_close(got, ref, tol, what):
+    assert got.shape == ref.shape and got.dtype == ref.dtype, what
+    if got.dtype.kind == "i":
+        assert np.array_equal(got, ref), what
+        return
+    scale = max(float(np.abs(ref).max()) if ref.size else 0.0, 1e-300)
+    err = float(np.abs(got.astype(np.float64) - ref.astype(np.float64)).max()) if ref.size else 0.0
+    assert err <= tol * scale, f"{what}: max |diff| {err:.3e} > {tol:g} * {scale:.3e}"
+
+
+def check_against_oracle(name, tensors, row_ptr, num_rows, num_cols, dtype):
+    ir = graphs.get(name)
+    ref_outs, ref_after = run_oracle(ir, tensors, row_ptr, num_rows, num_cols, THREADS)
+    outs, after = gpu_launch(name, tensors, row_ptr, num_rows, num_cols)
+    assert len(outs) == len(ref_outs)
+    tol = TOL.get(np.dtype(dtype), 0)
+    for spec, o, r in zip(ir.outputs, outs, ref_outs):
+        assert_close(o, r, tol, f"{name} output {spec['name']}")
+    for k in ref_after:                      # in-place map ops write through the inputs
+        assert_close(after[k], ref_after[k], tol, f"{name} input {k} after the call")
+    return outs
+
+
+REDUCER_GRAPHS = ["csr_spmv", "spmv_dot", "spring_mass", "swe_rusanov", "system_two_selectors"]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("structure", STRUCTURES)
+@pytest.mark.parametrize("name", REDUCER_GRAPHS)
+def test_reducer_graphs_on_every_row_structure(name, structure, dtype):
+    rng = np.random.default_rng(abs(hash((name, structure))) % 2**31)
+    row_ptr = row_structure(structure, rng)
+    tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get(name), dtype, rng, row_ptr=row_ptr)
+    print(f"case {name} {structure} {np.dtype(dtype).name} rows={nr} ne={ne}", flush=True)
+    check_against_oracle(name, tensors, row_ptr, nr, nc, dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("structure", ["mesh", "skewed", "mostly_empty"])
+def test_every_map_op(structure, dtype):
+    rng = np.random.default_rng(21)
+    row_ptr = row_structure(structure, rng)
+    ne, nr = int(row_ptr[-1]), len(row_ptr) - 1
+    t = op_zoo_inputs(rng, ne, max(nr, 64), dtype)
+    print(f"case op_zoo {structure} {np.dtype(dtype).name}", flush=True)
+    check_against_oracle("op_zoo", t, row_ptr, nr, max(nr, 64), dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("ne", [1, 255, 2048, 100003])
+def test_flat_graphs(ne, dtype):
+    rng = np.random.default_rng(ne)
+    for name in ("mass_sum", "map_store"):
+        tensors, _, nr, nc, _ = make_inputs(graphs.get(name), dtype, rng, ne=ne)
+        print(f"case {name} ne={ne} {np.dtype(dtype).name}", flush=True)
+        check_against_oracle(name, tensors, None, nr, nc, dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.int64, np.float64])
+def test_index_shuffle_map_only_int64(dtype):
+    rng = np.random.default_rng(3)
+    tensors, _, nr, nc, ne = make_inputs(graphs.get("bpoints_copy"), dtype, rng, ne=77777)
+    outs = check_against_oracle("bpoints_copy", tensors, None, nr, nc, dtype)
+    assert outs == []
+    _, after = gpu_launch("bpoints_copy", tensors, None, nr, nc)
+    assert np.array_equal(after["bp_1"], tensors["bpoints"][:, 1])
+
+
+def test_results_are_bitwise_reproducible():
+    rng = np.random.default_rng(9)
+    row_ptr = row_structure("skewed", rng)
+    tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get("spmv_dot"), np.float32, rng, row_ptr=row_ptr)
+    a, _ = gpu_launch("spmv_dot", tensors, row_ptr, nr, nc)
+    for _ in range(3):
+        b, _ = gpu_launch("spmv_dot", tensors, row_ptr, nr, nc)
+        assert all(np.array_equal(x, y) for x, y in zip(a, b))
+
+
+# ---------------------------------------------------------------------------------------------
+# the five benchmark workloads at oracle-friendly sizes
+# ---------------------------------------------------------------------------------------------
+def test_workload_1_laplacian_2d_fp32():
+    w = W.laplacian_2d_spmv(256)
+    assert (w.num_rows, w.ne, w.algorithmic_bytes) == (65536, 326656, 3399684)
+    (y,), _ = gpu_launch(w.graph, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols)
+    (ref,), _ = run_oracle(graphs.get(w.graph), w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, THREADS)
+    A = sp.csr_matrix((np.abs(w.tensors["vals"]).astype(np.float64), w.tensors["selector_idx"], w.row_end_offsets))
+    row_scale = A @ np.abs(w.tensors["x"]).astype(np.float64)
+    assert np.all(np.abs(y.astype(np.float64) - ref) <= 1e-5 * np.maximum(np.abs(ref), row_scale))
+
+
+def test_workload_2_spring_mass_fp32():
+    w = W.spring_mass_grid(40)
+    check_against_oracle(w.graph, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, np.float32)
+
+
+def test_workload_3_shallow_water_fp64():
+    w = W.shallow_water_mesh(60000)
+    check_against_oracle(w.graph, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, np.float64)
+    m = W.mass_sum_of(w)
+    check_against_oracle(m.graph, m.tensors, None, m.num_rows, m.num_cols, np.float64)
+
+
+def test_workload_4_rmat_fp32():
+    w = W.rmat_spmv(16)
+    (y,), _ = gpu_launch(w.graph, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols)
+    (ref,), _ = run_oracle(graphs.get(w.graph), w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, THREADS)
+    assert np.all(np.abs(y - ref) <= 1e-5 * np.abs(ref))      # all terms positive: the row scale is |ref|
+    assert np.all(y[np.diff(w.row_end_offsets) == 0] == 0)
+
+
+def test_workload_5_poisson_fp64():
+    w = W.poisson_3d_spmv_dot(64)
+    check_against_oracle(w.graph, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, np.float64)
+
+
+# ---------------------------------------------------------------------------------------------
+# full benchmark sizes: size-independent properties instead of the oracle
+# ---------------------------------------------------------------------------------------------
+def test_poisson_256_cubed_stencil_and_dot():
+    w = W.poisson_3d_spmv_dot(256)
+    ext = load_named(w.graph, build_if_missing=False)
+    args = W.launch_arguments(w, ext.param_names(), "cuda")
+    y, dot = ext.merged_spmv_launch(*args)
+    x = args[ext.param_names().index("x")].view(256, 256, 256)
+    ref = 6 * x.clone()
+    ref[1:] -= x[:-1]; ref[:-1] -= x[1:]
+    ref[:, 1:] -= x[:, :-1]; ref[:, :-1] -= x[:, 1:]
+    ref[:, :, 1:] -= x[:, :, :-1]; ref[:, :, :-1] -= x[:, :, 1:]
+    assert (y.view_as(ref) - ref).abs().max().item() <= 1e-12 * 12
+    d_ref = (x * ref).sum().item()
+    assert abs(dot.item() - d_ref) <= 1e-12 * abs(d_ref)
+
+
+def test_rmat_scale_20_linearity_and_library_product():
+    w = W.rmat_spmv(20)
+    ext = load_named(w.graph, build_if_missing=False)
+    names = ext.param_names()
+    args = W.launch_arguments(w, names, "cuda")
+    (y1,) = ext.merged_spmv_launch(*args)
+    xi = names.index("x")
+    x1 = args[xi]
+    x2 = torch.rand_like(x1)
+    args[xi] = x2
+    (y2,) = ext.merged_spmv_launch(*args)
+    args[xi] = (0.5 * x1 + 2.0 * x2).contiguous()
+    (y3,) = ext.merged_spmv_launch(*args)
+    scale = (0.5 * y1 + 2.0 * y2).abs().max().item()
+    assert (y3 - (0.5 * y1 + 2.0 * y2)).abs().max().item() <= 1e-5 * scale
+    A = torch.sparse_csr_tensor(args[names.index("row_end_offsets")].long(), args[names.index("selector_idx")].long(),
+                                args[names.index("vals")].double(), size=(w.num_rows, w.num_cols))
+    ref = (A @ x1.double().unsqueeze(1)).squeeze(1)
+    assert ((y1.double() - ref).abs() <= 1e-5 * ref.abs()).all()
+
+
+# ---------------------------------------------------------------------------------------------
+# error behaviour of the call surface (TORCH_CHECK -> RuntimeError in the reference)
+# ---------------------------------------------------------------------------------------------
+def test_argument_checks_raise_runtime_error():
+    w = W.laplacian_2d_spmv(16)
+    ext = load_named(w.graph, build_if_missing=False)
+    names = ext.param_names()
+    good = W.launch_arguments(w, names, "cuda")
+
+    def call(**replace):
+        a = list(good)
+        for k, v in replace.items():
+            a[names.index(k)] = v
+        return ext.merged_spmv_launch(*a)
+
+    with pytest.raises(RuntimeError, match="CUDA"):
+        call(vals=good[names.index("vals")].cpu())
+    with pytest.raises(RuntimeError, match="x dtype mismatch"):
+        call(x=good[names.index("x")].double())
+    with pytest.raises(RuntimeError, match="selector_idx dtype mismatch"):
+        call(selector_idx=good[names.index("selector_idx")].long())
+    with pytest.raises(RuntimeError, match="contiguous"):
+        call(x=torch.stack([good[names.index("x")]] * 2, dim=1)[:, 0])
+    with pytest.raises(RuntimeError, match="non-empty"):
+        call(selector_idx=good[names.index("selector_idx")][:0])
+    with pytest.raises(RuntimeError, match="Unsupported dtype"):
+        call(vals=good[names.index("vals")].half())
+    with pytest.raises(RuntimeError, match="num_rows \\+ 1"):
+        call(row_end_offsets=good[names.index("row_end_offsets")][:-1].contiguous())
+    with pytest.raises(RuntimeError, match="takes"):
+        ext.merged_spmv_launch(*good, 1)
+    (y,) = ext.merged_spmv_launch(**dict(zip(names, good)))          # keyword names are registered too
+    assert y.shape == (w.num_rows,)

@@ -1,0 +1,171 @@
+"""Host-side logic and the C interface of the generated libraries (no GPU needed)."""
+import ctypes
+import json
+import os
+import re
+
+import pytest
+
+from flexspmv_amd import build, graphs
+from flexspmv_amd.binding import ABI_VERSION, EXPORTED_SYMBOLS, LaunchArgs, load_library
+from flexspmv_amd.codegen.merged_gen_binding import binding_plan, generate_binding_code
+from flexspmv_amd.codegen.merged_gen_gpu import analyse, generate_hip_source
+from flexspmv_amd.ir import GraphBuilder, get_dim_length
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _lib(name):
+    ir = graphs.get(name)
+    path = build.library_path(ir)
+    if not build.is_current(ir):
+        path = build.compile_graph(ir)     # hipcc cross-compiles without a GPU
+    return load_library(path)
+
+
+# ---------------------------------------------------------------------------------------------
+# binding contract: argument order equals the generated bindings the reference keeps in its tree
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["system_two_selectors", "bpoints_copy"])
+def test_binding_order_matches_reference_generated_binding(name, golden_dir):
+    with open(os.path.join(golden_dir, "binding_fixtures.json")) as f:
+        gold = json.load(f)[name]
+    ir = graphs.get(name)
+    sig = generate_binding_code(None, ir.inputs, ir.outputs, ir.selector_register)
+    assert [p["name"] for p in sig["params"]] == gold["params"]
+    assert [{k: o[k] for k in ("name", "kind", "dim")} for o in sig["outputs"]] == gold["outputs"]
+    assert sig["dispatch_tensor"] == gold["dispatch_tensor"]
+    assert sig["allow_int64"] == gold["allow_int64"]
+
+
+def test_binding_groups():
+    plan = binding_plan(*graphs.get("spring_mass").six()[:3])
+    assert plan.non_gather_value_inputs == ["k", "rest"]
+    assert plan.gather_value_inputs == ["pos"]
+    assert plan.selector_inputs == ["gather_src", "gather_dst"]
+    assert [(o.name, o.kind, o.dim) for o in plan.outputs] == [("scatter", "reducer", 3), ("sum_1", "sum", 1)]
+    # a selector module used twice contributes one index tensor
+    b = GraphBuilder("twice")
+    b.placeholder("v", (2,)); b.placeholder("w", (1,))
+    b.select("s_a", "v", module="sel"); b.select("s_b", "v", module="sel")
+    b.map("add", "add", ["s_a", "s_b"]); b.reduce("red", "add"); b.output("red")
+    assert binding_plan(*b.build().six()[:3]).selector_inputs == ["sel"]
+
+
+def test_shape_rule_and_unknown_op():
+    assert get_dim_length((2, 3)) == 6 and get_dim_length((1,)) == 1
+    b = GraphBuilder("bad")
+    b.placeholder("v", (1,))
+    with pytest.raises(ValueError, match="not supported"):
+        b.map("cosh", "c", ["v"])
+
+
+# ---------------------------------------------------------------------------------------------
+# generator: stage split, widths, policy
+# ---------------------------------------------------------------------------------------------
+def test_stage_split_of_row_aligned_selector():
+    kp = analyse(graphs.get("spmv_dot"))
+    assert kp.vars["mul"].stage == 1 and kp.vars["mul_1"].stage == 2 and kp.vars["selector_row"].stage == 2
+    assert (kp.xch_width, kp.red_width, kp.agg_width, kp.row_width) == (1, 1, 1, 1)
+    src, sig = generate_hip_source(graphs.get("spmv_dot"))
+    assert sig["row_aligned_index_inputs"] == ["selector_row_idx"]
+    assert "p.selector_row_ptr" not in src.split("static FLEX_DEV void fetch")[1]   # never dereferenced
+    kp = analyse(graphs.get("spring_mass"))
+    assert kp.row_width == 3 and kp.red_width == 3 and kp.agg_width == 1
+    assert kp.xch_width == 3 + 1 + 1            # gathered source position, k, rest cross into the walk
+
+
+def test_plain_spmv_exchanges_only_its_products():
+    kp = analyse(graphs.get("csr_spmv"))
+    assert (kp.xch_width, kp.row_width, kp.agg_width) == (1, 0, 0)
+    src, sig = generate_hip_source(graphs.get("csr_spmv"))
+    assert sig["policy"]["block"] == 256 and sig["policy"]["ipt"]["float64"] == 8
+    assert "STAGE1_PURE = true" in src and "STAGE2_PURE = true" in src
+
+
+def test_policy_shrinks_tile_for_wide_graphs():
+    _, sig = generate_hip_source(graphs.get("op_zoo"))
+    ipt = sig["policy"]["ipt"]
+    assert ipt["float64"] <= ipt["float32"] <= 8 and ipt["float64"] >= 1
+
+
+def test_generated_source_is_deterministic_and_hash_keyed():
+    a, _ = generate_hip_source(graphs.get("swe_rusanov"))
+    b, _ = generate_hip_source(graphs.get("swe_rusanov"))
+    assert a == b
+    ir = graphs.get("swe_rusanov")
+    assert ir.content_hash() in a and build.graph_dir(ir).endswith(ir.content_hash())
+
+
+def test_no_cuda_or_compat_layers_in_kernel_sources():
+    bad = re.compile(r"cub::|hipcub|rocprim|__HIP_PLATFORM|cuda_runtime|triton", re.I)
+    for fn in os.listdir(build.CSRC_DIR):
+        with open(os.path.join(build.CSRC_DIR, fn)) as f:
+            assert not bad.search(f.read()), fn
+
+
+# ---------------------------------------------------------------------------------------------
+# C interface: symbols, signature, argument validation (all before any GPU call)
+# ---------------------------------------------------------------------------------------------
+def test_header_symbols_are_exported_by_every_library():
+    with open(os.path.join(ROOT, "include", "flexspmv.h")) as f:
+        header = f.read()
+    declared = set(re.findall(r"\b(flexspmv_[a-z_]+)\s*\(", header))
+    assert declared == set(EXPORTED_SYMBOLS)
+    for name in graphs.REGISTRY:
+        lib = _lib(name)
+        for sym in declared:
+            assert getattr(lib, sym) is not None
+        assert lib.flexspmv_abi_version() == ABI_VERSION
+        sig = json.loads(lib.flexspmv_signature().decode())
+        assert sig["graph"] == name and sig["hash"] == graphs.get(name).content_hash()
+
+
+def _args(lib, **over):
+    sig = json.loads(lib.flexspmv_signature().decode())
+    nv, ni, no = len(sig["value_inputs"]), len(sig["index_inputs"]), len(sig["outputs"])
+    keep = []
+    def arr(n):
+        a = (ctypes.c_void_p * max(n, 1))(*([0x1000] * max(n, 1)))
+        keep.append(a)
+        return ctypes.cast(a, ctypes.POINTER(ctypes.c_void_p))
+    la = LaunchArgs()
+    la.struct_size = ctypes.sizeof(LaunchArgs)
+    la.dtype = 0
+    la.value_inputs, la.num_value_inputs = arr(nv), nv
+    la.index_inputs, la.num_index_inputs = arr(ni), ni
+    la.outputs, la.num_outputs = arr(no), no
+    la.row_end_offsets = 0x1000
+    la.num_rows, la.num_cols, la.ne = 10, 10, 30
+    la.workspace, la.workspace_bytes = 0, 0
+    for k, v in over.items():
+        setattr(la, k, v)
+    la._keep = keep
+    return la
+
+
+def test_launch_rejects_bad_arguments_without_touching_the_gpu():
+    lib = _lib("csr_spmv")
+    err = lambda: lib.flexspmv_last_error().decode()
+    assert lib.flexspmv_launch(None) == -1
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, struct_size=8))) == -1 and "struct_size" in err()
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, flags=1))) == -1
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, num_value_inputs=1))) == -1 and "counts" in err()
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, dtype=2))) == -2 and "Unsupported dtype" in err()
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, ne=0))) == -1 and "non-empty" in err()
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, num_rows=0))) == -1
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, ne=2**31 - 100))) == -3 and "2^31" in err()
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib))) == -4 and "workspace" in err()       # no scratch given
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, workspace=0x1000, workspace_bytes=1 << 20,
+                                                  row_end_offsets=0))) == -1 and "row_end_offsets" in err()
+
+
+def test_workspace_query():
+    lib = _lib("spmv_dot")
+    small = lib.flexspmv_workspace_bytes(1, 1000, 7000)
+    big = lib.flexspmv_workspace_bytes(1, 16777216, 117047296)
+    assert 0 < small < big < 64 << 20
+    assert lib.flexspmv_workspace_bytes(2, 1000, 7000) == 0          # int64 not compiled into this library
+    assert lib.flexspmv_workspace_bytes(1, 2**30, 2**30) == 0        # does not fit 32-bit offsets
+    flat = _lib("bpoints_copy")
+    assert flat.flexspmv_workspace_bytes(2, 100, 100) == 0           # map-only needs no scratch

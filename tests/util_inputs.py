@@ -1,0 +1,76 @@
+"""Seeded inputs for any sub-graph of flexspmv_amd.graphs, from its binding signature."""
+import numpy as np
+
+from flexspmv_amd.codegen.merged_gen_binding import generate_binding_code
+
+
+def row_structure(kind, rng, tile=2048):
+    """CSR row pointer of a named shape.  Shapes are chosen to hit every path of the reducer kernel."""
+    if kind == "mesh":            # 3..7 per row: row path
+        lens = rng.integers(3, 8, 5000)
+    elif kind == "mesh_with_gaps":  # short rows and empty rows mixed: row path, open rows at tile ends
+        lens = rng.integers(0, 9, 7000)
+    elif kind == "skewed":        # empty rows, long rows spanning several tiles: merge path + carry runs
+        lens = (rng.pareto(1.2, 3000) * 3).astype(np.int64)
+        lens[rng.random(3000) < 0.35] = 0
+        lens[100] = 3 * tile + 17
+        lens[101] = 0
+        lens[2000] = tile
+    elif kind == "one_long_row":  # a single row far longer than a tile: every tile carries into it
+        lens = np.array([0, 0, 9 * tile + 5, 0])
+    elif kind == "mostly_empty":  # > 512 row ends in a tile: merge path with direct stores
+        lens = (rng.random(20000) < 0.05).astype(np.int64) * rng.integers(1, 40, 20000)
+        lens[-1] = 7
+    elif kind == "tiny":
+        lens = np.array([1])
+    elif kind == "exact_tiles":   # rows + nnz is a multiple of the tile
+        lens = np.full(512, 7)
+    elif kind == "len33":         # one row just over the row-path limit inside regular rows
+        lens = np.full(900, 5)
+        lens[450] = 33
+    else:
+        raise ValueError(kind)
+    if lens.sum() == 0:
+        lens[-1] = 1
+    return np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+
+
+STRUCTURES = ["mesh", "mesh_with_gaps", "skewed", "one_long_row", "mostly_empty", "tiny", "exact_tiles", "len33"]
+
+
+def make_inputs(ir, dtype, rng, row_ptr=None, ne=None, positive=True):
+    """(tensors, row_ptr, num_rows, num_cols, ne) for a sub-graph.  Gather sources get
+    max(num_rows, 64) rows so that row-aligned selectors index them safely."""
+    sig = generate_binding_code(None, ir.inputs, ir.outputs, ir.selector_register)
+    if sig["has_reducer"]:
+        assert row_ptr is not None
+        num_rows, ne = len(row_ptr) - 1, int(row_ptr[-1])
+    else:
+        num_rows = ne
+    nv = max(num_rows, 64)
+    row_aligned = {s["selector_name"] + "_idx" for s in ir.selector_register if s.get("row_aligned")}
+    lo, hi = (0.5, 2.0) if positive else (-1.0, 1.0)
+    tensors = {}
+    for name in sig["non_gather_value_inputs"]:
+        d = sig["value_dims"][name]
+        tensors[name] = _values(rng, (ne, d) if d > 1 else (ne,), dtype, lo, hi)
+    for name in sig["gather_value_inputs"]:
+        d = sig["value_dims"][name]
+        tensors[name] = _values(rng, (nv, d) if d > 1 else (nv,), dtype, lo, hi)
+    for name in sig["index_inputs"]:
+        if name in row_aligned and sig["has_reducer"]:
+            tensors[name] = np.repeat(np.arange(num_rows, dtype=np.int32), np.diff(row_ptr)).astype(np.int32)
+        elif sig["has_reducer"]:
+            # never the edge's own row: keeps distances in the mesh maps away from an exact 0 / 0
+            rows = np.repeat(np.arange(num_rows, dtype=np.int64), np.diff(row_ptr))
+            tensors[name] = ((rows + 1 + rng.integers(0, nv - 1, ne)) % nv).astype(np.int32)
+        else:
+            tensors[name] = rng.integers(0, nv, ne).astype(np.int32)
+    num_cols = nv if sig["gather_value_inputs"] else ne
+    return tensors, row_ptr, num_rows, num_cols, ne
+
+
+def _values(rng, shape, dtype, lo, hi):
+    if np.dtype(dtype).kind == "i":
+        return rng.integers(-1000, 1000, shape).astype(dtype)
+    return rng.uniform(lo, hi, shape).astype(dtype)
