@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused merge-path SpMV / map + reducer + aggregator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--size N] [--all]
+
+A step is one ``merged_spmv_launch`` of the workload's fused sub-graph (all kernels of the launch,
+inputs resident in HBM).  The headline workload is the 3-D 7-point Poisson operator on a 256^3 grid in
+float64: fused ``y = A x`` and ``x . y``.  One JSON line is printed:
+
+* ``value``         effective GB/s = algorithmic bytes per step / wall time per step over K steps
+                    (every streamed array once, every gathered source once, every output once)
+* ``roofline``      the dominant kernel alone: algorithmic bytes / its mean duration, measured with HIP
+                    events around that kernel on the launch stream, against the 8 TB/s HBM peak
+* ``cpu_baseline``  the CPU oracle (a port of the reference's OpenMP path) on the same inputs, timed on
+                    this host's cores, and the parity of the GPU result against it
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+DEFAULT_SIZE = {"poisson3d": 256, "rmat": 22, "spring_mass": 100, "shallow_water": 1_000_000, "laplacian2d": 256}
+DTYPE_TAG = {"float32": "f32", "float64": "f64", "int64": "i64"}
+
+
+def host_threads() -> int:
+    n = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    if n <= 0:
+        n = os.cpu_count() or 1
+    return max(1, min(n, 256))          # 256 = size of the reference's per-thread carry arrays
+
+
+def time_workload(w, steps, warmup):
+    """GPU leg: returns (result dict, outputs of the last launch as numpy arrays)."""
+    import numpy as np
+    import torch
+
+    from flexspmv_amd import graphs
+    from flexspmv_amd import workloads as W
+    from flexspmv_amd.binding import load_named
+
+    ext = load_named(w.graph, build_if_missing=False)
+    args = W.launch_arguments(w, ext.param_names(), "cuda:0")
+    outs = None
+    for _ in range(max(warmup, 1)):
+        outs = ext.merged_spmv_launch(*args)
+    torch.cuda.synchronize()
+
+    # whole steps: K launches between two synchronisations
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        outs = ext.merged_spmv_launch(*args)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    # the dominant kernel alone: HIP events recorded around it inside the library, on the launch stream
+    ext.time_kernel = True
+    kernel_ms = []
+    for _ in range(steps):
+        ext.merged_spmv_launch(*args)
+        kernel_ms.append(ext.last_kernel_ms())
+    ext.time_kernel = False
+    kernel_ms_mean = sum(kernel_ms) / len(kernel_ms)
+
+    result = {
+        "workload": w.name, "graph": w.graph, "dtype": str(next(iter(w.tensors.values())).dtype),
+        "ne": int(w.ne), "num_rows": int(w.num_rows), "algorithmic_bytes": int(w.algorithmic_bytes),
+        "flops": int(w.flops), "ms_per_step": ms_per_step, "kernel_ms": kernel_ms_mean,
+        "kernel_ms_min": min(kernel_ms),
+        "gbs": w.algorithmic_bytes / ms_per_step / 1e6, "kernel_gbs": w.algorithmic_bytes / kernel_ms_mean / 1e6,
+        "edges_per_s": w.ne / ms_per_step * 1e3, "gflops": w.flops / ms_per_step / 1e6,
+        "policy": ext.signature["policy"],
+    }
+
+    result["output_kinds"] = [o["kind"] for o in ext.signature["outputs"]]
+    return result, [o.cpu().numpy() for o in outs]
+
+
+def cpu_leg(w, result, outs, cpu_runs):
+    """CPU leg, run after every GPU timing is done (its OpenMP threads would otherwise disturb the
+    launch thread): times the oracle on the same inputs and checks the GPU outputs against it."""
+    import numpy as np
+
+    from flexspmv_amd import graphs
+    if cpu_runs > 0:
+        from oracle.runner import run_oracle
+        T = host_threads()
+        ir = graphs.get(w.graph)
+        ref = None
+        times = []
+        for i in range(cpu_runs + 1):
+            c0 = time.perf_counter()
+            ref, _ = run_oracle(ir, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, T)
+            if i > 0:
+                times.append(time.perf_counter() - c0)
+        times.sort()
+        cpu_ms = times[len(times) // 2] * 1e3
+        tol = 1e-5 if result["dtype"] == "float32" else 1e-12
+        # Aggregators in float32: the reference sums millions of terms sequentially per thread, so its
+        # own result drifts from the exact sum by far more than the tolerance (and depends on the
+        # thread count).  They are therefore checked against the same oracle evaluated in float64.
+        ref_hi = None
+        if result["dtype"] == "float32" and "sum" in result["output_kinds"]:
+            hi = {k: (v.astype(np.float64) if v.dtype == np.float32 else v) for k, v in w.tensors.items()}
+            ref_hi, _ = run_oracle(ir, hi, w.row_end_offsets, w.num_rows, w.num_cols, T)
+        worst = 0.0
+        for i, (o, r) in enumerate(zip(outs, ref)):
+            if ref_hi is not None and result["output_kinds"][i] == "sum":
+                r = ref_hi[i]
+            o = o.astype(np.float64)
+            scale = max(float(np.abs(r).max()), 1e-300)
+            worst = max(worst, float(np.abs(o - r.astype(np.float64)).max()) / scale)
+        result["cpu"] = {"ms": cpu_ms, "gbs": w.algorithmic_bytes / cpu_ms / 1e6, "threads": T,
+                         "max_rel_diff_vs_gpu": worst, "tolerance": tol, "parity_ok": bool(worst <= tol)}
+    return result
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="poisson3d", choices=sorted(DEFAULT_SIZE))
+    ap.add_argument("--size", type=int, default=None, help="grid edge / R-MAT scale / point count")
+    ap.add_argument("--all", action="store_true", help="also time the other four workloads (extra JSON key)")
+    ap.add_argument("--cpu-runs", type=int, default=5, help="timed runs of the CPU baseline (0 = skip)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists for it)",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    from flexspmv_amd import workloads as W
+
+    size = a.size if a.size is not None else DEFAULT_SIZE[a.workload]
+    w = W.WORKLOADS[a.workload](size)
+    head, head_outs = time_workload(w, a.steps, a.warmup)
+    torch.cuda.empty_cache()
+    pending = []
+    if a.all:
+        for name in ("rmat", "spring_mass", "shallow_water", "laplacian2d"):
+            if name == a.workload:
+                continue
+            wo = W.WORKLOADS[name](DEFAULT_SIZE[name])
+            r, o = time_workload(wo, a.steps, a.warmup)
+            torch.cuda.empty_cache()
+            pending.append((name, wo, r, o))
+    head = cpu_leg(w, head, head_outs, a.cpu_runs)
+    others = {}
+    if pending:
+        for name, wo, r, o in pending:
+            r = cpu_leg(wo, r, o, min(a.cpu_runs, 3))
+            others[name] = {k: r[k] for k in ("workload", "dtype", "ne", "num_rows", "algorithmic_bytes",
+                                              "ms_per_step", "kernel_ms", "gbs", "kernel_gbs", "edges_per_s",
+                                              "gflops")}
+            others[name]["frac_of_hbm_peak"] = r["kernel_gbs"] / HBM_PEAK_GBS
+            if "cpu" in r:
+                others[name]["cpu"] = r["cpu"]
+
+    line = {
+        "metric": "fused SpMV effective HBM GB/s (% of MI355X peak) + edges/sec, 1 GPU",
+        "value": head["gbs"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": DTYPE_TAG[head["dtype"]],
+        "data": "synthetic",
+        "config": {"workload": f"{head['workload']} fused y=A*x and x.y ({head['graph']})", "ne": head["ne"],
+                   "num_rows": head["num_rows"], "algorithmic_bytes": head["algorithmic_bytes"],
+                   "policy": head["policy"]},
+        "pct_of_hbm_peak": 100.0 * head["gbs"] / HBM_PEAK_GBS,
+        "edges_per_s": head["edges_per_s"],
+        "gflops": head["gflops"],
+        "roofline": {"bound": "hbm", "achieved": head["kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["kernel_gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "flex::reduce_kernel" if head["graph"] not in ("mass_sum", "map_store", "bpoints_copy")
+                     else "flex::flat_kernel",
+                     "kernel_ms": head["kernel_ms"]},
+    }
+    if "cpu" in head:
+        c = head["cpu"]
+        line["cpu_baseline"] = {"value": c["gbs"], "unit": "GB/s", "cores": c["threads"], "kind": "port",
+                                "sample": f"the whole workload ({head['workload']}), median of {a.cpu_runs} runs "
+                                          f"after one warm-up, {c['ms']:.1f} ms per run",
+                                "ms": c["ms"], "parity_max_rel_diff": c["max_rel_diff_vs_gpu"],
+                                "parity_tolerance": c["tolerance"], "parity_ok": c["parity_ok"]}
+    if others:
+        line["other_workloads"] = others
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

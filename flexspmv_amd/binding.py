@@ -27,10 +27,11 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 from . import build as _build
 from .ir import FusedGraphIR
 
-ABI_VERSION = 1
+ABI_VERSION = 2
+FLAG_TIME_KERNEL = 1
 DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
 EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
-                    "flexspmv_last_error", "flexspmv_abi_version")
+                    "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms")
 
 
 class LaunchArgs(ctypes.Structure):
@@ -59,6 +60,13 @@ def load_library(path: str) -> ctypes.CDLL:
     """dlopen a generated library and type its five entry points."""
     if not os.path.exists(path):
         raise RuntimeError(f"FlexSpmv library {path} is not built (run __graft_entry__.build())")
+    try:
+        # torch ships its own HIP runtime; it has to be the one already in the process when a generated
+        # library (linked against libamdhip64 by soname) is opened, or the two runtimes disagree about
+        # the device
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = ctypes.CDLL(path, mode=ctypes.RTLD_LOCAL)
     lib.flexspmv_launch.argtypes = [ctypes.POINTER(LaunchArgs)]
     lib.flexspmv_launch.restype = ctypes.c_int
@@ -68,6 +76,8 @@ def load_library(path: str) -> ctypes.CDLL:
     lib.flexspmv_signature.restype = ctypes.c_char_p
     lib.flexspmv_last_error.argtypes = []
     lib.flexspmv_last_error.restype = ctypes.c_char_p
+    lib.flexspmv_last_kernel_ms.argtypes = [ctypes.POINTER(ctypes.c_float)]
+    lib.flexspmv_last_kernel_ms.restype = ctypes.c_int
     lib.flexspmv_abi_version.argtypes = []
     lib.flexspmv_abi_version.restype = ctypes.c_int
     if lib.flexspmv_abi_version() != ABI_VERSION:
@@ -98,6 +108,7 @@ class HipExtension:
         self._dtypes = set(self.signature["dtypes"])
         self._param_names = [p["name"] for p in self.signature["params"]]
         self._workspace: Dict[Any, Any] = {}
+        self.time_kernel = False   # set True to bracket the dominant kernel of each launch with events
 
     # -- helpers -------------------------------------------------------------------------
     def param_names(self) -> List[str]:
@@ -193,6 +204,7 @@ class HipExtension:
         la.row_end_offsets = ro.data_ptr()
         la.num_rows, la.num_cols, la.ne = num_rows, num_cols, ne
         la.workspace, la.workspace_bytes = ws.data_ptr(), ws.numel()
+        la.flags = FLAG_TIME_KERNEL if self.time_kernel else 0
         with torch.cuda.device(device):
             la.stream = torch.cuda.current_stream(device).cuda_stream
             rc = self._lib.flexspmv_launch(ctypes.byref(la))
@@ -203,6 +215,14 @@ class HipExtension:
         return tuple(outs)
 
     __call__ = merged_spmv_launch
+
+    def last_kernel_ms(self) -> float:
+        """Duration of the dominant kernel of the last launch made with ``time_kernel = True``."""
+        ms = ctypes.c_float(0.0)
+        rc = self._lib.flexspmv_last_kernel_ms(ctypes.byref(ms))
+        if rc != 0:
+            raise RuntimeError(f"flexspmv_last_kernel_ms failed ({rc}): {self._lib.flexspmv_last_error().decode()}")
+        return float(ms.value)
 
 
 def load_extension(ir: FusedGraphIR, build_if_missing: bool = True) -> HipExtension:

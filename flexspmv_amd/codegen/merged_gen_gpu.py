@@ -474,6 +474,7 @@ extern "C" {{
 int flexspmv_abi_version(void) {{ return FLEXSPMV_ABI_VERSION; }}
 const char* flexspmv_signature(void) {{ return kSignature; }}
 const char* flexspmv_last_error(void) {{ return flex::g_last_error; }}
+int flexspmv_last_kernel_ms(float* ms) {{ return flex::last_kernel_ms(ms); }}
 
 size_t flexspmv_workspace_bytes(int32_t dtype, int64_t num_rows, int64_t ne) {{
   switch (dtype) {{

@@ -26,6 +26,24 @@ inline int fail_hip(hipError_t e, const char* where) {
   return (int)e;
 }
 
+// HIP events that bracket the dominant kernel of a launch made with FLEXSPMV_FLAG_TIME_KERNEL.
+struct KernelTimer {
+  hipEvent_t start = nullptr, stop = nullptr;
+  bool armed = false;
+  bool ready() {
+    if (start == nullptr && (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess)) return false;
+    return true;
+  }
+};
+inline thread_local KernelTimer g_timer;
+inline int last_kernel_ms(float* ms) {
+  if (ms == nullptr || !g_timer.armed) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "no timed launch on this thread");
+  hipError_t e = hipEventSynchronize(g_timer.stop);
+  if (e == hipSuccess) e = hipEventElapsedTime(ms, g_timer.start, g_timer.stop);
+  if (e != hipSuccess) return fail_hip(e, "reading kernel timer");
+  return FLEXSPMV_OK;
+}
+
 constexpr size_t align_up(size_t n, size_t a = 256) { return (n + a - 1) / a * a; }
 constexpr int FIXUP_BLOCK = 256;
 constexpr int MAX_PERSISTENT_BLOCKS = 8192;  // upper bound used to size the aggregator partials
@@ -109,6 +127,8 @@ struct Dispatch {
       return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "row_end_offsets is required by a reducer sub-graph");
 
     hipStream_t stream = (hipStream_t)a->stream;
+    const bool timed = (a->flags & FLEXSPMV_FLAG_TIME_KERNEL) != 0 && g_timer.ready();
+    g_timer.armed = false;
     char* ws = (char*)a->workspace;
     V* partials = (V*)(ws + l.off_partials);
     const int nnz = (int)a->ne;
@@ -123,8 +143,10 @@ struct Dispatch {
       const int search_blocks = (l.num_tiles + 1 + 255) / 256;
       hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(256), 0, stream, l.num_tiles, TILE,
                          row_end, num_rows, nnz, coords);
+      if (timed) (void)hipEventRecord(g_timer.start, stream);
       hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid_for_tiles(l.num_tiles)), dim3(BLOCK), 0, stream,
                          p, row_end, num_rows, nnz, (const int2*)coords, l.num_tiles, carry_row, carry_val, partials);
+      if (timed) g_timer.armed = (hipEventRecord(g_timer.stop, stream) == hipSuccess);
       V* block_partials = (V*)(ws + l.off_block_partials);
       hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, BLOCK / WAVE>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0, stream, p,
                          l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials, block_partials);
@@ -135,8 +157,10 @@ struct Dispatch {
     } else {
       int grid = resident_grid(flat_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
       if (grid > l.num_tiles) grid = l.num_tiles;
+      if (timed) (void)hipEventRecord(g_timer.start, stream);
       hipLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream, p, nnz,
                          l.num_tiles, partials);
+      if (timed) g_timer.armed = (hipEventRecord(g_timer.stop, stream) == hipSuccess);
       if (G::AGG_WIDTH > 0) {
         hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
                            (const V*)partials, grid);
@@ -152,7 +176,7 @@ inline int check_counts(const flexspmv_launch_args* a, int nv, int ni, int no) {
   if (a == nullptr) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "args is NULL");
   if (a->struct_size != sizeof(flexspmv_launch_args))
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "struct_size does not match this library's flexspmv_launch_args");
-  if (a->flags != 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "flags must be 0");
+  if ((a->flags & ~FLEXSPMV_FLAG_TIME_KERNEL) != 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "unknown bits in flags");
   if (a->num_value_inputs != nv || a->num_index_inputs != ni || a->num_outputs != no)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "argument counts do not match flexspmv_signature()");
   if ((nv > 0 && a->value_inputs == nullptr) || (ni > 0 && a->index_inputs == nullptr) ||

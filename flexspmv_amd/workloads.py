@@ -131,7 +131,8 @@ def rmat_spmv(scale: int = 22, degree: int = 16, dtype="float32", seed: int = 4,
 # spring-mass on a jittered grid
 # ---------------------------------------------------------------------------------------------
 def spring_mass_grid(n: int = 100, dtype="float32", seed: int = 2) -> Workload:
-    """Workload 2: n^3 vertices, 6-neighbour springs as half-edges sorted by destination vertex."""
+    """Workload 2: n^3 vertices displaced by U(-0.1, 0.1) h from a regular lattice, 6-neighbour springs
+    (rest length = lattice spacing h) as half-edges sorted by destination vertex."""
     dtype = np.dtype(dtype)
     rng = np.random.default_rng(seed)
     V = n ** 3
@@ -147,9 +148,8 @@ def spring_mass_grid(n: int = 100, dtype="float32", seed: int = 2) -> Workload:
     sa, sb = np.concatenate(a_list), np.concatenate(b_list)
     S = len(sa)
     k_spring = rng.uniform(0.5, 2.0, S).astype(dtype)
-    rest = np.linalg.norm(pos[sa].astype(np.float64) - pos[sb].astype(np.float64), axis=1).astype(dtype)
-    # rest length = initial length gives zero force; perturb the positions afterwards so forces are non-trivial
-    pos = (pos + (rng.uniform(-0.02, 0.02, (V, 3)) * h).astype(dtype)).astype(dtype)
+    # springs are at rest on the regular lattice (length h); the jitter above is the displacement
+    rest = np.full(S, h, dtype=dtype)
     dst = np.concatenate([sa, sb]); src = np.concatenate([sb, sa])
     kk = np.concatenate([k_spring, k_spring]); ll = np.concatenate([rest, rest])
     order = np.lexsort((src, dst))

@@ -17,6 +17,9 @@
  *                             (codegen/merged_gen_binding.py:27-78,112-134); here it is data.
  *   flexspmv_last_error       the strings TORCH_CHECK raises (cuda_template/merged_binding_template.cu:40-50).
  *   flexspmv_abi_version      no counterpart; lets a loader reject a stale library.
+ *   flexspmv_last_kernel_ms   the GpuTimer bracket of the reference's CUDA harness
+ *                             (src/flex_spmv_full_red.cu:298-330, utils.h:634-669), narrowed to the
+ *                             dominant kernel of one launch so that a roofline can be measured live.
  */
 #ifndef FLEXSPMV_H_
 #define FLEXSPMV_H_
@@ -28,7 +31,10 @@
 extern "C" {
 #endif
 
-#define FLEXSPMV_ABI_VERSION 1
+#define FLEXSPMV_ABI_VERSION 2
+
+/* flexspmv_launch_args.flags */
+#define FLEXSPMV_FLAG_TIME_KERNEL 1u /* bracket the dominant kernel with HIP events on args->stream */
 
 /* Value types a library may have been generated for (flexspmv_launch_args.dtype). */
 enum flexspmv_dtype { FLEXSPMV_F32 = 0, FLEXSPMV_F64 = 1, FLEXSPMV_I64 = 2 };
@@ -73,7 +79,7 @@ typedef struct flexspmv_launch_args {
   void* workspace;
   size_t workspace_bytes;
   void* stream;
-  uint32_t flags; /* reserved, must be 0 */
+  uint32_t flags; /* 0 or FLEXSPMV_FLAG_* */
 } flexspmv_launch_args;
 
 /* Run the fused sub-graph once.  Returns FLEXSPMV_OK, a negative flexspmv_status, or a hipError_t. */
@@ -88,6 +94,12 @@ const char* flexspmv_signature(void);
 
 /* Message of the last failed call on this thread ("" if none). */
 const char* flexspmv_last_error(void);
+
+/* Duration in milliseconds of the dominant kernel (the reducer kernel, or the flat kernel of an
+ * aggregator / map-only library) of the calling thread's most recent flexspmv_launch that carried
+ * FLEXSPMV_FLAG_TIME_KERNEL.  Blocks until that kernel has finished.  Returns FLEXSPMV_OK, or
+ * FLEXSPMV_ERR_BAD_ARGUMENT when no such launch was made. */
+int flexspmv_last_kernel_ms(float* ms);
 
 /* FLEXSPMV_ABI_VERSION the library was built against. */
 int flexspmv_abi_version(void);

@@ -59,8 +59,18 @@ def check_against_oracle(name, tensors, row_ptr, num_rows, num_cols, dtype):
     outs, after = gpu_launch(name, tensors, row_ptr, num_rows, num_cols)
     assert len(outs) == len(ref_outs)
     tol = TOL.get(np.dtype(dtype), 0)
-    for spec, o, r in zip(ir.outputs, outs, ref_outs):
-        assert_close(o, r, tol, f"{name} output {spec['name']}")
+    # float32 aggregators: the reference adds every edge sequentially per thread, so its own result
+    # drifts from the exact sum by up to (edges per thread) * eps; the centre of the comparison is the
+    # same oracle evaluated in float64 on the same inputs
+    ref_hi = None
+    if np.dtype(dtype) == np.float32 and any(o["target"] == "sum" for o in ir.outputs):
+        hi = {k: (v.astype(np.float64) if v.dtype == np.float32 else v) for k, v in tensors.items()}
+        ref_hi, _ = run_oracle(ir, hi, row_ptr, num_rows, num_cols, THREADS)
+    for i, (spec, o, r) in enumerate(zip(ir.outputs, outs, ref_outs)):
+        if ref_hi is not None and spec["target"] == "sum":
+            assert_close(o.astype(np.float64), ref_hi[i], tol, f"{name} aggregator {spec['name']} vs float64 oracle")
+        else:
+            assert_close(o, r, tol, f"{name} output {spec['name']}")
     for k in ref_after:                      # in-place map ops write through the inputs
         assert_close(after[k], ref_after[k], tol, f"{name} input {k} after the call")
     return outs
@@ -135,7 +145,7 @@ def test_workload_1_laplacian_2d_fp32():
 
 
 def test_workload_2_spring_mass_fp32():
-    w = W.spring_mass_grid(40)
+    w = W.spring_mass_grid(100)
     check_against_oracle(w.graph, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, np.float32)
 
 
