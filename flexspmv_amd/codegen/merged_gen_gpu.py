@@ -51,6 +51,7 @@ class KernelPlan:
     row_sources: List[Tuple[str, str, int, int]]  # (selector var, source tensor, dim, first slot)
     red_slices: List[Tuple[str, int, int]]    # (reducer name, first slot, dim)
     agg_slices: List[Tuple[str, int, int]]
+    op_stage: Dict[int, int] = field(default_factory=dict)   # index into map_operations -> stage
     xch_width: int = 0
     red_width: int = 0
     agg_width: int = 0
@@ -68,7 +69,22 @@ def _literal(a: Any) -> str:
 
 
 def analyse(ir: FusedGraphIR) -> KernelPlan:
-    """Variable table, stage split and LDS slot assignment for a sub-graph."""
+    """Variable table, stage split and LDS slot assignment for a sub-graph.
+
+    A ``row_aligned`` selector may be served from the merge path (no index array read, its dependants
+    run in the walk) or like any other selector (index array read, everything runs in the coalesced
+    stage).  The first is taken only when it does not widen the per-edge LDS exchange: for ``y = A x``
+    with ``x . y`` it saves the 4-byte index per edge for free, for the mesh maps it would push every
+    input through LDS and shrink the tile.
+    """
+    with_rows = _analyse(ir, use_row_aligned=True)
+    if with_rows.row_width == 0:
+        return with_rows
+    plain = _analyse(ir, use_row_aligned=False)
+    return with_rows if with_rows.xch_width <= plain.xch_width else plain
+
+
+def _analyse(ir: FusedGraphIR, use_row_aligned: bool) -> KernelPlan:
     inputs, outputs, selector_register, map_ops, red_ops, agg_ops = ir.six()
     plan = binding_plan(inputs, outputs, selector_register)
     has_reducer = bool(red_ops)
@@ -77,7 +93,7 @@ def analyse(ir: FusedGraphIR) -> KernelPlan:
     cur_stage: Dict[str, int] = {}   # stage a variable's current value lives in (in-place ops may raise it)
     for s in selector_register:
         dim = get_dim_length(s["shape"])
-        stage = 2 if (s.get("row_aligned") and has_reducer and s["selector"] == 1) else 1
+        stage = 2 if (use_row_aligned and s.get("row_aligned") and has_reducer and s["selector"] == 1) else 1
         var = s["name"] if s["selector"] == 1 else s["selector_name"]
         vars[var] = Var(var, "tensor", dim, f"TensorInput_{s['target']}_T", stage)
         cur_stage[var] = stage
@@ -96,7 +112,8 @@ def analyse(ir: FusedGraphIR) -> KernelPlan:
     # reducer arguments take the first slots so that a plain SpMV exchanges exactly its products
     red_arg_names = [arg_name(r["args"][0]) for r in red_ops]
 
-    for op in map_ops:
+    op_stage: Dict[int, int] = {}
+    for op_index, op in enumerate(map_ops):
         o = op["op"]
         if o in ("reducer", "sum"):
             continue
@@ -104,7 +121,7 @@ def analyse(ir: FusedGraphIR) -> KernelPlan:
                                       [op["args"][0]] + ([op["args"][2]] if o == "setitem" else []))]
         used = [a for a in args if isinstance(a, str) and a in vars]
         stage = max([1] + [cur_stage[a] for a in used]) if has_reducer else 1
-        op["_stage"] = stage
+        op_stage[op_index] = stage
         if stage == 2:
             for a in used:
                 if vars[a].stage == 1:
@@ -149,12 +166,12 @@ def analyse(ir: FusedGraphIR) -> KernelPlan:
     row_sources: List[Tuple[str, str, int, int]] = []
     row_width = 0
     for s in selector_register:
-        if s["selector"] == 1 and vars[s["name"]].stage == 2 and s.get("row_aligned"):
+        if s["selector"] == 1 and vars[s["name"]].stage == 2 and s.get("row_aligned") and use_row_aligned:
             dim = get_dim_length(s["shape"])
             row_sources.append((s["name"], s["target"], dim, row_width))
             row_width += dim
 
-    return KernelPlan(plan, vars, exchange, row_sources, red_slices, agg_slices,
+    return KernelPlan(plan, vars, exchange, row_sources, red_slices, agg_slices, op_stage=op_stage,
                       xch_width=len(exchange), red_width=red_width, agg_width=agg_width,
                       row_width=row_width)
 
@@ -240,7 +257,7 @@ def _indent(lines: Sequence[str], n: int = 4) -> str:
 
 def _choose_ipt(kp: KernelPlan, value_bytes: int) -> int:
     """Items per thread so that one block's LDS stays inside LDS_BUDGET_BYTES."""
-    per_item = value_bytes * (max(kp.xch_width, 1) + kp.row_width)
+    per_item = value_bytes * max(kp.xch_width, 1)
     for ipt in (8, 4, 2, 1):
         if BLOCK_THREADS * ipt * per_item <= LDS_BUDGET_BYTES:
             return ipt
@@ -321,11 +338,11 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         s2 += [f"{sel}.values[{i}] = rv.v[{first + i}];" for i in range(dim)]
 
     map_output_names = {o.name: o for o in plan.outputs if o.kind == "map"}
-    for op in map_ops:
+    for op_index, op in enumerate(map_ops):
         o = op["op"]
         if o in ("reducer", "sum"):
             continue
-        stage = op.get("_stage", 1) if has_reducer else 1
+        stage = kp.op_stage.get(op_index, 1) if has_reducer else 1
         body = s1 if stage == 1 else s2
         body.extend(_emit_map(op, kp.vars, "e"))
         if op["name"] in map_output_names:
@@ -384,7 +401,7 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         "hash": ir.content_hash(),
         "dtypes": list(dtypes),
         "row_aligned_index_inputs": sorted({s["selector_name"] + "_idx" for s in selector_register
-                                            if s.get("row_aligned") and has_reducer}),
+                                            if s["selector"] == 1 and kp.vars[s["name"]].stage == 2}),
         "policy": {"block": block, "ipt": {k: ipt[k] for k in dtypes}},
         "widths": {"exchange": kp.xch_width, "reduce": kp.red_width, "aggregate": kp.agg_width,
                    "row": kp.row_width},
@@ -498,9 +515,6 @@ int flexspmv_launch(const flexspmv_launch_args* a) {{
             print("Stage-1 code: ", line)
         for line in s2:
             print("Stage-2 code: ", line)
-    # the analysis annotates ops with '_stage'; leave the caller's lists as they were
-    for op in map_ops:
-        op.pop("_stage", None)
     return src, signature
 
 

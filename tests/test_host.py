@@ -70,9 +70,11 @@ def test_stage_split_of_row_aligned_selector():
     src, sig = generate_hip_source(graphs.get("spmv_dot"))
     assert sig["row_aligned_index_inputs"] == ["selector_row_idx"]
     assert "p.selector_row_ptr" not in src.split("static FLEX_DEV void fetch")[1]   # never dereferenced
+    # the mesh maps would have to push every input through LDS: their row selector is read like any other
     kp = analyse(graphs.get("spring_mass"))
-    assert kp.row_width == 3 and kp.red_width == 3 and kp.agg_width == 1
-    assert kp.xch_width == 3 + 1 + 1            # gathered source position, k, rest cross into the walk
+    assert kp.row_width == 0 and kp.red_width == 3 and kp.agg_width == 1 and kp.xch_width == 3
+    _, sig = generate_hip_source(graphs.get("spring_mass"))
+    assert sig["row_aligned_index_inputs"] == []
 
 
 def test_plain_spmv_exchanges_only_its_products():
