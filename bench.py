@@ -132,6 +132,9 @@ def main() -> int:
     ap.add_argument("--size", type=int, default=None, help="grid edge / R-MAT scale / point count")
     ap.add_argument("--all", action="store_true", help="also time the other four workloads (extra JSON key)")
     ap.add_argument("--cpu-runs", type=int, default=5, help="timed runs of the CPU baseline (0 = skip)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain elementwise copies (dst = src + 1) of 1 GiB, a kernel of known "
+                         "traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists for it)",
@@ -148,6 +151,14 @@ def main() -> int:
     w = W.WORKLOADS[a.workload](size)
     head, head_outs = time_workload(w, a.steps, a.warmup)
     torch.cuda.empty_cache()
+    if a.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").fill_(1.0)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1.0, out=dst)   # one elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     pending = []
     if a.all:
         for name in ("rmat", "spring_mass", "shallow_water", "laplacian2d"):
