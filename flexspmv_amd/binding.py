@@ -29,6 +29,7 @@ from .ir import FusedGraphIR
 
 ABI_VERSION = 2
 FLAG_TIME_KERNEL = 1
+FLAG_REUSE_TILES = 2
 DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
 EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
                     "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms")
@@ -109,6 +110,11 @@ class HipExtension:
         self._param_names = [p["name"] for p in self.signature["params"]]
         self._workspace: Dict[Any, Any] = {}
         self.time_kernel = False   # set True to bracket the dominant kernel of each launch with events
+        # Reuse of the tile table between launches on the same, unmodified row_end_offsets tensor (the
+        # reference's wrapper keeps it as an immutable buffer, dynamic_replace_submodule.py:118-137).
+        # Off by default: every launch then does all the work a launch of the reference does.
+        self.reuse_tiles = False
+        self._tile_key = None
 
     # -- helpers -------------------------------------------------------------------------
     def param_names(self) -> List[str]:
@@ -205,6 +211,11 @@ class HipExtension:
         la.num_rows, la.num_cols, la.ne = num_rows, num_cols, ne
         la.workspace, la.workspace_bytes = ws.data_ptr(), ws.numel()
         la.flags = FLAG_TIME_KERNEL if self.time_kernel else 0
+        if self.reuse_tiles and self._has_reducer:
+            key = (ro.data_ptr(), ro._version, num_rows, ne, dt, ws.data_ptr(), str(device))
+            if key == self._tile_key:
+                la.flags |= FLAG_REUSE_TILES
+            self._tile_key = key
         with torch.cuda.device(device):
             la.stream = torch.cuda.current_stream(device).cuda_stream
             rc = self._lib.flexspmv_launch(ctypes.byref(la))

@@ -68,15 +68,48 @@ __device__ __forceinline__ int2 merge_path_search(int diag, const int* __restric
   return make_int2(min(lo, num_rows), diag - lo);
 }
 
+// The same coordinate with fewer dependent loads.  g(i) = row_end[i] + i + 1 is strictly increasing and
+// the answer is the first i with g(i) > diag, so any probe sequence that keeps the bracket valid gives
+// the identical result.  A few Newton-like probes (step = residual / average slope of g) land within
+// a handful of rows when row lengths are regular; the bisection that follows bounds the cost when
+// they are not.  The search is pure latency (about 25 dependent loads for 16 M rows), so fewer probes
+// is what counts.
+__device__ __forceinline__ int2 merge_path_search_interp(int diag, const int* __restrict__ row_end, int num_rows,
+                                                         int nnz) {
+  int lo = max(diag - nnz, 0);
+  int hi = min(diag, num_rows);
+  const float inv_slope = (float)num_rows / ((float)num_rows + (float)nnz);  // rows per merge item
+  int p = (int)((float)diag * inv_slope);
+#pragma unroll 1
+  for (int it = 0; it < 4 && hi - lo > 4; ++it) {
+    p = min(max(p, lo), hi - 1);
+    const int gp = row_end[p] + p + 1;
+    if (gp <= diag) lo = p + 1;
+    else hi = p;
+    p += (int)((float)(diag - gp) * inv_slope) + (gp <= diag ? 1 : 0);
+  }
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (row_end[mid] <= diag - mid - 1) lo = mid + 1;
+    else hi = mid;
+  }
+  return make_int2(min(lo, num_rows), diag - lo);
+}
+
 // One search per tile boundary: coords[t] is where tile t starts, coords[num_tiles] where the path ends.
 __global__ void __launch_bounds__(256)
 tile_search_kernel(int num_tiles, int tile_items, const int* __restrict__ row_end, int num_rows, int nnz,
-                   int2* __restrict__ coords) {
+                   int2* __restrict__ coords, unsigned* __restrict__ ticket) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t == 0) *ticket = 0u;  // arms fixup_kernel's last-block detection
   if (t > num_tiles) return;
   const long long d = (long long)t * tile_items;
   const int diag = (int)min(d, (long long)num_rows + nnz);
+#ifdef FLEX_TUNE_BISECTION_ONLY  // tuning switch: the reference's plain bisection
   coords[t] = merge_path_search(diag, row_end, num_rows, nnz);
+#else
+  coords[t] = merge_path_search_interp(diag, row_end, num_rows, nnz);
+#endif
 }
 
 // Which tile a block works on.  By default tile = block: neighbouring tiles run at the same time on
@@ -520,17 +553,18 @@ flat_kernel(const typename G::Params p, const int nnz, const int num_tiles,
 }
 
 // ----------------------------------------------------------------------------------------------
-// Fix-up: fold tile carries into their rows (tile order) and pre-reduce the aggregator partials.
+// Fix-up: fold tile carries into their rows (tile order) and finish the aggregators.
 // Block b handles tiles [b*BLOCK, (b+1)*BLOCK): a thread owns the carry of one tile and, when it is
 // the first tile of a run that carries into the same row, adds the whole run to that row.  The
 // block's aggregator partials (PARTS_PER_TILE per tile, one per wavefront of the reducer block) are
-// summed in a fixed order into block_partials[b].
+// summed in a fixed order into block_partials[b]; the block that finishes last adds the blocks'
+// partials, again in a fixed order, and assigns the outputs (no floating-point atomics anywhere).
 // ----------------------------------------------------------------------------------------------
 template <class G, int BLOCK, int PARTS_PER_TILE>
 __global__ void __launch_bounds__(BLOCK)
 fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restrict__ carry_row,
              const typename G::Value* __restrict__ carry_val, const typename G::Value* __restrict__ agg_partials,
-             typename G::Value* __restrict__ block_partials) {
+             typename G::Value* __restrict__ block_partials, unsigned* __restrict__ ticket) {
   using V = typename G::Value;
   constexpr int RED = G::RED_WIDTH, AGG = G::AGG_WIDTH;
   constexpr int NW = BLOCK / WAVE;
@@ -567,12 +601,49 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
       for (int c = 0; c < AGG; ++c) s_wave_agg[threadIdx.x / WAVE][c] = acc.v[c];
     }
     __syncthreads();
+    __shared__ bool s_is_last;
     if (threadIdx.x == 0) {
 #pragma unroll
       for (int c = 0; c < AGG; ++c) {
         V s = s_wave_agg[0][c];
         for (int w = 1; w < NW; ++w) s += s_wave_agg[w][c];
-        block_partials[(size_t)blockIdx.x * AGG + c] = s;
+        __hip_atomic_store(&block_partials[(size_t)blockIdx.x * AGG + c], s, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      }
+      // The block that draws the last ticket sees every other block's partial: each block publishes
+      // its partial before taking a ticket (release), the last block acquires after taking its own.
+      __atomic_thread_fence(__ATOMIC_RELEASE);
+      const unsigned drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      s_is_last = (drawn == gridDim.x - 1);
+    }
+    __syncthreads();
+    if (s_is_last) {
+      __atomic_thread_fence(__ATOMIC_ACQUIRE);
+      // ordered final sum over the blocks' partials (same order on every run)
+      Pack<V, AGG> fin;
+      zero(fin);
+      for (int j = threadIdx.x; j < (int)gridDim.x; j += BLOCK) {
+#pragma unroll
+        for (int c = 0; c < AGG; ++c)
+          fin.v[c] += __hip_atomic_load(&block_partials[(size_t)j * AGG + c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      wave_sum_to_last_lane<V, AGG>(fin.v);
+      __syncthreads();  // s_wave_agg is reused
+      if ((threadIdx.x & (WAVE - 1)) == WAVE - 1) {
+#pragma unroll
+        for (int c = 0; c < AGG; ++c) s_wave_agg[threadIdx.x / WAVE][c] = fin.v[c];
+      }
+      __syncthreads();
+      if (threadIdx.x == 0) {
+        Pack<V, AGG> total;
+#pragma unroll
+        for (int c = 0; c < AGG; ++c) {
+          V s = s_wave_agg[0][c];
+          for (int w = 1; w < NW; ++w) s += s_wave_agg[w][c];
+          total.v[c] = s;
+        }
+        G::store_agg(p, total);
+        *ticket = 0u;  // re-armed for launches that reuse the tile table and skip the search kernel
       }
     }
   }

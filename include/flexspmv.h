@@ -35,6 +35,12 @@ extern "C" {
 
 /* flexspmv_launch_args.flags */
 #define FLEXSPMV_FLAG_TIME_KERNEL 1u /* bracket the dominant kernel with HIP events on args->stream */
+/* Skip the tile search: the caller guarantees that the previous launch of this library with this
+ * workspace completed, used the same dtype, num_rows, ne and the same, unmodified row_end_offsets, and
+ * that nothing else wrote to the workspace since.  The tile table left in the workspace by that launch
+ * is then reused (the reference recomputes it on every call, include/merged_spmv_kernels.cuh:60-99;
+ * a solver iterating on a fixed sparsity pattern needs it once). */
+#define FLEXSPMV_FLAG_REUSE_TILES 2u
 
 /* Value types a library may have been generated for (flexspmv_launch_args.dtype). */
 enum flexspmv_dtype { FLEXSPMV_F32 = 0, FLEXSPMV_F64 = 1, FLEXSPMV_I64 = 2 };
@@ -59,8 +65,9 @@ enum flexspmv_status {
  *   row_end_offsets  int32[num_rows + 1] with a leading 0 (CSR row pointer); ignored (may be NULL) by
  *                  libraries without a reducer.
  *   ne             number of edges (non-zeros); must be > 0.
- *   workspace      scratch of at least flexspmv_workspace_bytes(...) bytes, 256-byte aligned; contents
- *                  are not preserved between calls.
+ *   workspace      scratch of at least flexspmv_workspace_bytes(...) bytes, 256-byte aligned.  Its contents
+ *                  mean nothing to the caller; they only have to be left alone between two launches when
+ *                  the second one carries FLEXSPMV_FLAG_REUSE_TILES.
  *   stream         hipStream_t to launch on (NULL = default stream).  The call is asynchronous.
  */
 typedef struct flexspmv_launch_args {

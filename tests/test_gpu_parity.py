@@ -131,6 +131,39 @@ def test_results_are_bitwise_reproducible():
         assert all(np.array_equal(x, y) for x, y in zip(a, b))
 
 
+def test_tile_table_reuse_matches_full_launches():
+    """Launches that keep the tile table of the previous launch give the bits of a full launch; a
+    different row structure in between invalidates the table (the launcher notices and searches again)."""
+    rng = np.random.default_rng(17)
+    ext = load_named("spmv_dot", build_if_missing=False)
+
+    def arguments(structure):
+        row_ptr = row_structure(structure, rng)
+        tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get("spmv_dot"), np.float64, rng, row_ptr=row_ptr)
+        out = []
+        for pname in ext.param_names():
+            if pname == "row_end_offsets":
+                out.append(torch.from_numpy(row_ptr).cuda())
+            elif pname in ("num_rows", "num_cols"):
+                out.append(int(nr if pname == "num_rows" else nc))
+            else:
+                out.append(torch.from_numpy(np.ascontiguousarray(tensors[pname])).cuda())
+        return out
+
+    a_args, b_args = arguments("skewed"), arguments("mesh")
+    full_a = [o.clone() for o in ext.merged_spmv_launch(*a_args)]
+    full_b = [o.clone() for o in ext.merged_spmv_launch(*b_args)]
+    ext.reuse_tiles = True
+    try:
+        for args, full in ((a_args, full_a), (a_args, full_a), (a_args, full_a), (b_args, full_b),
+                           (b_args, full_b), (a_args, full_a)):
+            got = ext.merged_spmv_launch(*args)
+            torch.cuda.synchronize()
+            assert all(torch.equal(g, f) for g, f in zip(got, full))
+    finally:
+        ext.reuse_tiles = False
+
+
 # ---------------------------------------------------------------------------------------------
 # the five benchmark workloads at oracle-friendly sizes
 # ---------------------------------------------------------------------------------------------
