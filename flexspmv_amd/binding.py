@@ -106,6 +106,7 @@ class HipExtension:
         self._row_aligned = set(self.signature.get("row_aligned_index_inputs", []))
         self._outputs = self.signature["outputs"]
         self._has_reducer = bool(self.signature["has_reducer"])
+        self._streamed = set(self.signature["non_gather_value_inputs"])
         self._dtypes = set(self.signature["dtypes"])
         self._param_names = [p["name"] for p in self.signature["params"]]
         self._workspace: Dict[Any, Any] = {}
@@ -175,6 +176,9 @@ class HipExtension:
         dims = self.signature["value_dims"]
         for n, t in zip(self._value_names, values):
             _check(t.numel() % dims[n] == 0, f"{n}.numel() must be a multiple of its item width {dims[n]}")
+            # the kernels index a streamed tensor by edge id: a shorter one would be read out of bounds
+            if n in self._streamed:
+                _check(t.numel() >= ne * dims[n], f"{n} must hold one item of width {dims[n]} per edge ({ne})")
         if self._has_reducer:
             _check(ro.numel() == num_rows + 1, "row_end_offsets must have length num_rows + 1")
 

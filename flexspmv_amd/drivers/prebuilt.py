@@ -1,0 +1,47 @@
+"""The fused sub-graphs of the driver models, for building their libraries ahead of time.
+
+Sub-graph descriptions do not depend on mesh or lattice size (item shapes only), so the libraries built
+from small instances serve instances of any size."""
+from __future__ import annotations
+
+from typing import Callable, Dict, List
+
+import torch
+
+from .. import frontend as esr
+from ..ir import FusedGraphIR
+
+
+def _system(device="cpu", dtype=torch.float64):
+    from .system_model import make_system
+    return make_system(64, 17, 13, device=device, dtype=dtype)
+
+
+def _swe(device="cpu", dtype=torch.float64, points=900):
+    from .shallow_water import ShallowWaterEquation, synthetic_mesh
+    # time step well inside the stability limit of the mesh spacing (gravity wave speed is about 1)
+    return ShallowWaterEquation(synthetic_mesh(points, dtype=dtype, device=device),
+                                dt=min(0.002, 0.25 / points ** 0.5))
+
+
+def _spring(device="cpu", dtype=torch.float32, n=8):
+    from .spring_mass import SpringMass, lattice
+    pos, springs = lattice(n, dtype=dtype, device=device)
+    model = SpringMass(pos, springs)
+    with torch.no_grad():
+        model.pos.mul_(1.05)          # start 5 % stretched: the lattice breathes
+    return model
+
+
+MODELS: Dict[str, Callable[..., torch.nn.Module]] = {"system": _system, "swe": _swe, "spring": _spring}
+
+
+def model_graphs() -> List[FusedGraphIR]:
+    """Every sub-graph of every driver model that the generators implement."""
+    from ..python_wrapper.accelerate import lower_submodules
+    out: List[FusedGraphIR] = []
+    for name, factory in MODELS.items():
+        [compiled] = esr.compile([factory()], "torch")
+        irs, _ = lower_submodules(compiled, prefix=name)
+        out.extend(irs.values())
+    return out

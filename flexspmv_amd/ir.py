@@ -97,7 +97,9 @@ class FusedGraphIR:
         """Deterministic text form: the content key for build caches."""
         def clean(v):
             if isinstance(v, dict):
-                return {k: clean(x) for k, x in sorted(v.items()) if not k.startswith("_")}
+                # one library serves float32 and float64 alike: the two spell the same key
+                return {k: ("float" if k == "dtype_data" and str(x).endswith(("float32", "float64")) else clean(x))
+                        for k, x in sorted(v.items()) if not k.startswith("_")}
             if isinstance(v, (list, tuple)):
                 return [clean(x) for x in v]
             if isinstance(v, slice):

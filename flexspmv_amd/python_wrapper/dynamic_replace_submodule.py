@@ -1,0 +1,229 @@
+"""Swap a fused fx sub-module of a compiled model for a call into its generated library.
+
+Same surface as the reference (python_wrapper/dynamic_replace_submodule.py): ``get_submodules_wrapper``,
+``_coo_rows_to_csr_ptr``, ``_DynamicCudaWrapper`` and ``dynamic_replace_submodule(compiled_eqn, ext,
+submodule_name) -> bool``; ``ext`` is any object with ``merged_spmv_launch(<non-gather value tensors in
+placeholder order>, <gather sources in order of first use>, <one int32 index tensor per unique selector>,
+row_end_offsets, num_rows, num_cols)``.
+
+Deliberate differences:
+
+* selector index tensors are collected in the order in which the fused graph first calls each selector
+  module, which is the order the generated binding declares them in (codegen/merged_gen_binding.py:33-38);
+  the reference walks ``named_modules()`` and stops at the first Reducer
+  (dynamic_replace_submodule.py:65-72), which drops selectors registered after it;
+* the reducer's row ids must be sorted for the COO -> CSR conversion to describe them
+  (dynamic_replace_submodule.py:20-41 assumes it); unsorted ids raise instead of giving a wrong sum;
+* outputs are returned in the shapes the fused sub-module itself produces (``[n, 2, 1]`` stays that way).
+"""
+from __future__ import annotations
+
+from typing import Dict, Iterable, List, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from ..frontend.lite import Reducer, Selector
+
+
+def get_submodules_wrapper(eqn, node_name, run_to_collect=True):
+    """``[(fused sub-module, its call_module node)]`` for the node called ``node_name``."""
+    if run_to_collect:
+        eqn()
+    graph = eqn.jit_engine.graph
+    found = []
+    for node in graph.nodes:
+        if node.op == "call_module" and node.name == node_name:
+            found.append((eqn.get_submodule(node.target), node))
+    return found
+
+
+def _coo_rows_to_csr_ptr(row_ids: torch.Tensor, num_rows: Optional[int] = None) -> Tuple[torch.Tensor, int]:
+    """Sorted COO row ids -> CSR row pointer of length ``num_rows + 1`` (int64, device of ``row_ids``)."""
+    row_ids = row_ids.to(torch.int64)
+    if num_rows is None:
+        if row_ids.numel() == 0:
+            raise RuntimeError("row_ids is empty; cannot infer num_rows")
+        num_rows = int(row_ids.max().item()) + 1
+    if row_ids.numel() > 1 and bool((row_ids[1:] < row_ids[:-1]).any()):
+        raise RuntimeError("Reducer row ids must be sorted ascending for the CSR conversion; sort the edges "
+                           "by destination row first (flexspmv_amd.python_wrapper.edge_order)")
+    if row_ids.numel() and (int(row_ids.min()) < 0 or int(row_ids.max()) >= num_rows):
+        raise RuntimeError("Reducer row ids outside [0, num_rows)")
+    counts = torch.bincount(row_ids, minlength=num_rows)
+    crow = torch.zeros(num_rows + 1, dtype=torch.int64, device=row_ids.device)
+    torch.cumsum(counts, dim=0, out=crow[1:])
+    return crow, num_rows
+
+
+def _iter_placeholders_in_order(gm) -> List[str]:
+    return [n.name for n in gm.graph.nodes if n.op == "placeholder"]
+
+
+def _collect_selector_modules(gm) -> Tuple[List[Tuple[str, nn.Module]], Optional[nn.Module]]:
+    """(unique Selector modules in order of first call, the Reducer module or None)."""
+    selectors: List[Tuple[str, nn.Module]] = []
+    reducer_mod: Optional[nn.Module] = None
+    seen = set()
+    for node in gm.graph.nodes:
+        if node.op != "call_module":
+            continue
+        mod = gm.get_submodule(node.target)
+        if type(mod) is Selector and node.target not in seen:
+            seen.add(node.target)
+            selectors.append((node.target, mod))
+        elif type(mod) is Reducer:
+            if reducer_mod is None:
+                reducer_mod = mod
+            elif mod is not reducer_mod and not (mod.n == reducer_mod.n and torch.equal(mod.idx, reducer_mod.idx)):
+                raise RuntimeError("the Reducers of one fused sub-module must share one row structure")
+    return selectors, reducer_mod
+
+
+def _infer_gather_value_inputs(gm, selector_qnames: Iterable[str]) -> List[str]:
+    """Placeholders that are gathered through a selector, in order of first use."""
+    names: List[str] = []
+    wanted = set(selector_qnames)
+    for node in gm.graph.nodes:
+        if node.op == "call_module" and node.target in wanted:
+            for a in node.all_input_nodes:
+                if a.op == "placeholder" and a.name not in names:
+                    names.append(a.name)
+    return names
+
+
+def _written_inputs(gm) -> List[str]:
+    """Placeholders the fused graph stores into (``x[:] = v``, ``x.copy_(v)``, ``x.add_(v)``)."""
+    import operator
+    out = []
+    for node in gm.graph.nodes:
+        inplace = (node.op == "call_function" and node.target is operator.setitem) or \
+                  (node.op == "call_method" and node.target in ("copy_", "add_"))
+        if inplace and node.args and getattr(node.args[0], "op", None) == "placeholder":
+            out.append(node.args[0].name)
+    return out
+
+
+def _output_shapes(gm) -> List[Tuple[int, ...]]:
+    for node in gm.graph.nodes:
+        if node.op == "output":
+            returned = node.args[0] if isinstance(node.args[0], (list, tuple)) else [node.args[0]]
+            return [tuple(r.meta["flex_shape"]) if "flex_shape" in r.meta else () for r in returned]
+    return []
+
+
+class _DynamicCudaWrapper(nn.Module):
+    """Callable with the fused sub-module's placeholders; launches the library and returns a list."""
+
+    def __init__(self, ext_module, input_param_names: List[str], non_gather_value_inputs: List[str],
+                 gather_value_inputs: List[str], selector_idx_tensors: List[torch.Tensor],
+                 row_end_offsets: Optional[torch.Tensor], output_shapes: Optional[List[Tuple[int, ...]]] = None,
+                 written_inputs: Iterable[str] = ()) -> None:
+        super().__init__()
+        names: List[str] = []
+        for i, t in enumerate(selector_idx_tensors):
+            t = t.contiguous()
+            if t.dtype != torch.int32:
+                t = t.to(torch.int32)
+            self.register_buffer(f"selector_{i}_idx", t, persistent=False)
+            names.append(f"selector_{i}_idx")
+        reo = None
+        if row_end_offsets is not None:
+            reo = row_end_offsets.contiguous()
+            if reo.dtype != torch.int32:
+                if int(reo[-1]) >= 2 ** 31:
+                    raise RuntimeError("row_end_offsets does not fit 32-bit offsets")
+                reo = reo.to(torch.int32)
+        self.register_buffer("row_end_offsets", reo, persistent=False)
+        self._ext = ext_module
+        self._input_param_names = list(input_param_names)
+        self._non_gather_value_inputs = list(non_gather_value_inputs)
+        self._gather_value_inputs = list(gather_value_inputs)
+        self._selector_buf_names = names
+        self._output_shapes = list(output_shapes) if output_shapes is not None else None
+        self._written_inputs = set(written_inputs)
+        self._dummy_ro: Dict[torch.device, torch.Tensor] = {}
+
+    def _on(self, name: str, device) -> torch.Tensor:
+        t = getattr(self, name)
+        if t.device != device:       # moved once, then kept: launches must see one unchanged tensor
+            t = t.to(device)
+            setattr(self, name, t)
+        return t
+
+    def __call__(self, *args):
+        if len(args) != len(self._input_param_names):
+            raise RuntimeError(f"fused sub-module takes {len(self._input_param_names)} tensors, {len(args)} given")
+        for n, a in zip(self._input_param_names, args):
+            if n in self._written_inputs and not a.is_contiguous():
+                raise RuntimeError(f"{n} is written in place by the fused kernel and must be contiguous")
+        arg_map = {n: a.contiguous() for n, a in zip(self._input_param_names, args)}
+        device = next(iter(arg_map.values())).device
+
+        if self.row_end_offsets is not None:
+            ro = self._on("row_end_offsets", device)
+            num_rows = int(ro.numel() - 1)
+        else:
+            ro = self._dummy_ro.get(device)
+            if ro is None:          # no reducer: the binding still takes a tensor here
+                ro = torch.tensor([42], dtype=torch.int32, device=device)
+                self._dummy_ro[device] = ro
+            num_rows = None
+        gv = self._gather_value_inputs[0] if self._gather_value_inputs else self._non_gather_value_inputs[0]
+        num_cols = int(arg_map[gv].shape[0])
+        if num_rows is None:
+            num_rows = num_cols
+
+        call_args = [arg_map[n] for n in self._non_gather_value_inputs]
+        call_args += [arg_map[n] for n in self._gather_value_inputs]
+        call_args += [self._on(b, device) for b in self._selector_buf_names]
+        call_args += [ro, num_rows, num_cols]
+
+        outs = self._ext.merged_spmv_launch(*call_args)
+        if outs is None:
+            return []
+        outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+        if self._output_shapes is not None and len(self._output_shapes) == len(outs):
+            outs = [o.view(s) if s and o.numel() == _numel(s) else o for o, s in zip(outs, self._output_shapes)]
+        return outs
+
+
+def _numel(shape) -> int:
+    n = 1
+    for s in shape:
+        n *= int(s)
+    return n
+
+
+def build_wrapper(gm, ext) -> _DynamicCudaWrapper:
+    """The wrapper for one fused sub-module ``gm``."""
+    input_param_names = _iter_placeholders_in_order(gm)
+    selector_modules, reducer_mod = _collect_selector_modules(gm)
+    selector_idx_tensors = [mod.idx for _, mod in selector_modules]
+    if reducer_mod is not None:
+        row_end_offsets, _ = _coo_rows_to_csr_ptr(reducer_mod.idx, int(reducer_mod.n))
+    else:
+        row_end_offsets = None
+    gather_value_inputs = _infer_gather_value_inputs(gm, [q for q, _ in selector_modules])
+    non_gather_value_inputs = [n for n in input_param_names if n not in gather_value_inputs]
+    wrapper = _DynamicCudaWrapper(ext, input_param_names, non_gather_value_inputs, gather_value_inputs,
+                                  selector_idx_tensors, row_end_offsets, _output_shapes(gm), _written_inputs(gm))
+    names = getattr(ext, "param_names", None)
+    if callable(names):             # a library of this package knows its own argument list: cross-check
+        expected = non_gather_value_inputs + gather_value_inputs
+        declared = names()
+        n_idx = len(selector_idx_tensors)
+        if declared[:len(expected)] != expected or len(declared) != len(expected) + n_idx + 3:
+            raise RuntimeError(f"library arguments {declared} do not match the fused sub-module "
+                               f"({expected} + {n_idx} index tensors)")
+    return wrapper
+
+
+def dynamic_replace_submodule(compiled_eqn: nn.Module, ext, submodule_name) -> bool:
+    """Replace the fused sub-module called by node ``submodule_name`` with a launch of ``ext``."""
+    for gm, node in get_submodules_wrapper(compiled_eqn, submodule_name, run_to_collect=False):
+        if node.name != submodule_name:
+            continue
+        setattr(compiled_eqn, node.target, build_wrapper(gm, ext))
+        return True
+    return False

@@ -1,0 +1,263 @@
+"""Host-side tests of the modelling front end, the tracer and the replacement wrapper (no GPU).
+
+The fused sub-modules are executed three ways and must agree: the model run eagerly, the compiled model
+(fused torch sub-modules called in stage order), and the compiled model with its sub-modules replaced by
+an extension object backed by the CPU oracle - which checks the whole host path (trace -> six lists ->
+binding order -> wrapper arguments) without a device.
+"""
+import operator
+
+import numpy as np
+import pytest
+import torch
+
+from flexspmv_amd import frontend as esr
+from flexspmv_amd import graphs
+from flexspmv_amd.codegen.merged_gen_binding import binding_plan
+from flexspmv_amd.drivers import ab_check
+from flexspmv_amd.drivers.prebuilt import MODELS
+from flexspmv_amd.drivers.shallow_water import ShallowWaterEquation, synthetic_mesh
+from flexspmv_amd.drivers.spring_mass import SpringMass, lattice
+from flexspmv_amd.drivers.system_model import make_system
+from flexspmv_amd.ir import FusedGraphIR
+from flexspmv_amd.python_wrapper import edge_order
+from flexspmv_amd.python_wrapper.accelerate import fused_call_nodes, lower_submodules
+from flexspmv_amd.python_wrapper.dynamic_replace_submodule import (_coo_rows_to_csr_ptr, _DynamicCudaWrapper,
+                                                                    dynamic_replace_submodule)
+from flexspmv_amd.trace.graph_trace import classify, trace_graph
+from oracle.runner import run_oracle
+
+
+class OracleExtension:
+    """``merged_spmv_launch`` of one sub-graph served by the CPU oracle (test double of a built library)."""
+
+    def __init__(self, ir: FusedGraphIR):
+        self.ir = ir
+        self.plan = binding_plan(ir.inputs, ir.outputs, ir.selector_register)
+        self.calls = 0
+
+    def param_names(self):
+        return [n for n, _ in self.plan.bind_params]
+
+    def merged_spmv_launch(self, *args):
+        self.calls += 1
+        bound = dict(zip(self.param_names(), args))
+        tensors = {k: v.detach().numpy() for k, v in bound.items() if isinstance(v, torch.Tensor)
+                   and k != "row_end_offsets"}
+        ro = bound["row_end_offsets"].numpy() if self.ir.has_reducer else None
+        outs, after = run_oracle(self.ir, tensors, ro, bound["num_rows"], bound["num_cols"], num_threads=3)
+        for k, v in after.items():           # in-place map ops write through the inputs
+            bound[k].detach().view(-1)[:] = torch.from_numpy(v).view(-1)
+        return tuple(torch.from_numpy(o) for o in outs) if outs else None
+
+
+def replace_all_with_oracle(compiled, prefix):
+    irs, skipped = lower_submodules(compiled, prefix)
+    exts = {}
+    for name, ir in irs.items():
+        exts[name] = OracleExtension(ir)
+        assert dynamic_replace_submodule(compiled, exts[name], name)
+    return exts, skipped
+
+
+def test_system_model_fuses_into_the_sub_graph_the_reference_generates():
+    [compiled] = esr.compile([make_system()], "torch")
+    names = [n.name for n in fused_call_nodes(compiled)]
+    assert len(names) == 2 and names[0].endswith("select_reduce") and names[1].endswith("map")
+    six = trace_graph(compiled.get_submodule(names[0]), compiled)
+    ref = graphs.get("system_two_selectors")
+    strip = lambda ops: [(o["name"], o["op"], tuple(o["shape"]), [str(a) for a in o["args"]]) for o in ops]  # noqa: E731
+    assert strip(six[3]) == strip(ref.map_operations)
+    assert strip(six[4]) == strip(ref.reducer_operations)
+    key = lambda s: (s["name"], s["target"], s["selector"], s["selector_name"], tuple(s["shape"]))  # noqa: E731
+    assert sorted(map(key, six[2])) == sorted(map(key, ref.selector_register))
+    assert [(o["name"], o["target"]) for o in six[1]] == [("reducer_1", "reducer")]
+    assert {i["name"] for i in six[0]} == {i["name"] for i in ref.inputs}
+
+
+@pytest.mark.parametrize("name", sorted(MODELS))
+def test_compiled_model_equals_eager_model(name):
+    eager, traced = MODELS[name](), MODELS[name]()
+    [compiled] = esr.compile([traced], "torch")
+    for _ in range(4):
+        eager()
+        compiled()
+    for (k, a), (_, b) in zip(eager.named_parameters(), traced.named_parameters()):
+        assert torch.equal(a, b), k
+
+
+def test_swe_groups_and_row_alignment():
+    [compiled] = esr.compile([MODELS["swe"]()], "torch")
+    nodes = fused_call_nodes(compiled)
+    kinds = [n.name.split("_", 1)[1] for n in nodes]
+    # per Runge-Kutta stage: interior faces, wall faces, one flat cell update; plus the final update
+    assert kinds.count("select_reduce") == 8 and kinds.count("map") == 5
+    irs, skipped = lower_submodules(compiled, "swe")
+    assert not skipped
+    interior = irs[nodes[0].name]
+    assert len(interior.reducer_operations) == 3
+    aligned = [s for s in interior.selector_register if s.get("row_aligned")]
+    assert aligned and all(s["selector_name"] == "gather_dst" for s in aligned)
+
+
+def test_read_after_write_and_write_after_read_keep_program_order():
+    class Chain(esr.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = esr.Tensor(torch.arange(8.0))
+            self.b = esr.Tensor(torch.ones(8))
+            self.c = esr.Tensor(torch.zeros(8))
+            self.pick = esr.Selector(torch.tensor([7, 6, 5, 4, 3, 2, 1, 0]))
+
+        def forward(self):
+            g = self.pick(self.a)         # reads a ...
+            self.a[:] = self.b * 2.0      # ... before it is overwritten
+            self.c[:] = self.a + g        # reads the new a
+            self.b.add_(self.c)           # and the next step sees the new b
+
+    eager, traced = Chain(), Chain()
+    [compiled] = esr.compile([traced], "torch")
+    for _ in range(3):
+        eager()
+        compiled()
+    for k in ("a", "b", "c"):
+        assert torch.equal(getattr(eager, k), getattr(traced, k)), k
+
+
+def test_operations_are_classified_by_identity_not_by_text():
+    import torch.fx as fx
+
+    def padded_where_thing(x):     # the text of this target contains 'add' and 'where'
+        return x
+
+    g = fx.Graph()
+    x = g.placeholder("x")
+    bad = g.call_function(padded_where_thing, (x,))
+    good = g.call_function(torch.where, (x, x, x))
+    ia = g.call_method("add_", (x, x))
+    with pytest.raises(ValueError, match="not supported"):
+        classify(bad)
+    assert classify(good) == "where" and classify(ia) == "add_"
+    assert classify(g.call_function(operator.truediv, (1.0, x))) == "truediv"
+
+
+def test_broadcast_along_the_edge_dimension_is_rejected_not_generated():
+    class Scaled(esr.Module):
+        def __init__(self):
+            super().__init__()
+            self.v = esr.Tensor(torch.rand(16))
+            self.total = esr.Tensor(torch.zeros(1))
+            self.out = esr.Tensor(torch.zeros(16))
+
+        def forward(self):
+            self.total[:] = esr.sum(self.v)
+            self.out[:] = self.v / self.total     # [16] / [1]
+
+    [compiled] = esr.compile([Scaled()], "torch")
+    irs, skipped = lower_submodules(compiled, "scaled")
+    assert any("different lengths" in why for why in skipped.values())
+    compiled()                                     # the torch sub-modules still run
+    assert torch.allclose(compiled.out.sum(), torch.tensor(1.0))
+
+
+@pytest.mark.parametrize("name,steps,tol", [("system", 2, 1e-14), ("spring", 3, 2e-5), ("swe", 2, 1e-12)])
+def test_replaced_model_matches_original_through_the_wrapper(name, steps, tol):
+    eager, traced = MODELS[name](), MODELS[name]()
+    [compiled] = esr.compile([traced], "torch")
+    exts, skipped = replace_all_with_oracle(compiled, f"t_{name}")
+    assert not skipped
+    for _ in range(steps):
+        eager()
+        compiled()
+    assert all(e.calls == steps for e in exts.values())
+    want, got = ab_check.save_state(eager), ab_check.save_state(traced)
+    if name == "system":
+        # (2,1) + (2,3): the reference's value type pairs flat element k of the wide operand with element
+        # k % 2 of the narrow one (data_struct_shared.cuh:611-636), torch pairs it with element k // 3.
+        # The generated code follows the reference, so this one tensor differs from torch by design.
+        narrow = (traced.selector_1(traced.vector_x) + traced.selector_2(traced.vector_x)).reshape(-1, 2)
+        k = torch.arange(6)
+        expected = narrow[:, k % 2] + traced.spm_2.reshape(-1, 6)
+        assert torch.allclose(got.pop("y_add_2").reshape(-1, 6), expected, rtol=1e-14, atol=0)
+        assert not torch.allclose(want.pop("y_add_2").reshape(-1, 6), expected)
+    worst, ok = ab_check.compare_states(want, got, tol)
+    assert ok, worst
+
+
+def test_wrapper_argument_order_and_shapes():
+    [compiled] = esr.compile([make_system(30, 9, 7)], "torch")
+    node = fused_call_nodes(compiled)[0]
+    seen = {}
+
+    class Probe:
+        def merged_spmv_launch(self, *args):
+            seen["args"] = args
+            return (torch.zeros(7, 2),)
+
+    assert dynamic_replace_submodule(compiled, Probe(), node.name)
+    assert not dynamic_replace_submodule(compiled, Probe(), "no_such_node")
+    wrapper = getattr(compiled, node.target)
+    assert isinstance(wrapper, _DynamicCudaWrapper)
+    compiled()
+    a = seen["args"]
+    # non-gather values in placeholder order, the gather source, two int32 index tensors, CSR, sizes
+    assert [tuple(t.shape) for t in a[:5]] == [(30, 2, 1), (30, 2, 3), (30, 2, 1), (30, 2, 3), (9, 2, 1)]
+    assert a[5].dtype == a[6].dtype == a[7].dtype == torch.int32
+    assert a[7].numel() == 8 and int(a[7][-1]) == 30 and a[8:] == (7, 9)
+    # the result is handed back in the shape the fused sub-module produces
+    assert tuple(compiled.y_reducer_1.shape) == (7, 2, 1)
+
+
+def test_coo_to_csr_and_unsorted_rows():
+    rows = torch.tensor([0, 0, 2, 2, 2, 5])
+    ptr, n = _coo_rows_to_csr_ptr(rows, 7)
+    assert n == 7 and ptr.tolist() == [0, 2, 2, 5, 5, 5, 6, 6]
+    assert _coo_rows_to_csr_ptr(rows)[1] == 6
+    with pytest.raises(RuntimeError, match="sorted"):
+        _coo_rows_to_csr_ptr(torch.tensor([1, 0, 2]), 3)
+    with pytest.raises(RuntimeError, match="outside"):
+        _coo_rows_to_csr_ptr(torch.tensor([0, 3]), 3)
+    assert edge_order.coo_to_csr(rows, 7).dtype == torch.int32
+
+
+def test_edge_ordering_helpers():
+    g = torch.Generator().manual_seed(0)
+    dst = torch.randint(0, 10, (50,), generator=g)
+    w = torch.rand(50, 3, generator=g)
+    sorted_dst, perm, w2 = edge_order.sort_edges_by_row(dst, w)
+    assert bool((sorted_dst[1:] >= sorted_dst[:-1]).all()) and torch.equal(w2, w[perm])
+    # stable: equal rows keep their original order
+    for r in range(10):
+        p = perm[sorted_dst == r]
+        assert bool((p[1:] > p[:-1]).all())
+    a, b = torch.tensor([0, 1, 2]), torch.tensor([1, 2, 0])
+    s2, d2, sign, origin, w3 = edge_order.half_edges(a, b, torch.tensor([10.0, 20.0, 30.0]))
+    assert d2.tolist() == sorted(d2.tolist()) and len(d2) == 6
+    pairs = {(int(s), int(d)) for s, d in zip(s2, d2)}
+    assert pairs == {(0, 1), (1, 2), (2, 0), (1, 0), (2, 1), (0, 2)}
+    assert torch.equal(w3, torch.tensor([10.0, 20.0, 30.0])[origin])
+    assert all((sg > 0) == ((int(s), int(d)) in {(0, 1), (1, 2), (2, 0)}) for s, d, sg in zip(s2, d2, sign))
+
+
+def test_swe_conserves_mass():
+    mesh = synthetic_mesh(400)
+    m = ShallowWaterEquation(mesh, dt=0.002)
+    mass = float((m.h * m.area).sum())
+    for _ in range(10):
+        m()
+    assert abs(float((m.h * m.area).sum()) - mass) < 1e-13
+    assert float(m.uh.abs().max()) > 0          # the bump started to move
+
+
+def test_spring_energy_is_half_k_stretch_squared():
+    pos, springs = lattice(4, dtype=torch.float64)
+    m = SpringMass(pos, springs, stiffness=3.0)
+    with torch.no_grad():
+        m.pos.mul_(1.1)                          # stretch every spring by 10 %
+    a, b = springs[:, 0], springs[:, 1]
+    rest = (pos[a] - pos[b]).norm(dim=1)
+    m()
+    expected = float((0.5 * 3.0 * (0.1 * rest) ** 2).sum())
+    assert abs(float(m.energy) - expected) < 1e-12 * expected
+    # internal forces cancel
+    assert float(m.force.sum(dim=0).abs().max()) < 1e-12
