@@ -17,11 +17,11 @@ def _system(device="cpu", dtype=torch.float64):
     return make_system(64, 17, 13, device=device, dtype=dtype)
 
 
-def _swe(device="cpu", dtype=torch.float64, points=900):
+def _swe(device="cpu", dtype=torch.float64, points=900, dt=0.0005):
+    """``dt`` is a literal of the generated kernels (as every Python number of a model is): another value
+    means other libraries.  0.0005 is stable up to about 250k mesh points (gravity wave speed is ~1)."""
     from .shallow_water import ShallowWaterEquation, synthetic_mesh
-    # time step well inside the stability limit of the mesh spacing (gravity wave speed is about 1)
-    return ShallowWaterEquation(synthetic_mesh(points, dtype=dtype, device=device),
-                                dt=min(0.002, 0.25 / points ** 0.5))
+    return ShallowWaterEquation(synthetic_mesh(points, dtype=dtype, device=device), dt=dt)
 
 
 def _spring(device="cpu", dtype=torch.float32, n=8):
@@ -33,7 +33,21 @@ def _spring(device="cpu", dtype=torch.float32, n=8):
     return model
 
 
-MODELS: Dict[str, Callable[..., torch.nn.Module]] = {"system": _system, "swe": _swe, "spring": _spring}
+def _swe_parts(device="cpu", points=900):
+    from .shallow_water_assembly import MeshComponentsCollector, synthetic_topology
+    return MeshComponentsCollector(synthetic_topology(points, device=device))
+
+
+def _swe_init(device="cpu", dtype=torch.float64, points=900):
+    from .shallow_water_assembly import Initializer, MeshComponentsCollector, synthetic_topology
+    mesh = synthetic_topology(points, device=device)
+    parts = MeshComponentsCollector(mesh)
+    parts()
+    return Initializer(mesh, parts, dtype)
+
+
+MODELS: Dict[str, Callable[..., torch.nn.Module]] = {"system": _system, "swe": _swe, "spring": _spring,
+                                                     "swe_parts": _swe_parts, "swe_init": _swe_init}
 
 
 def model_graphs() -> List[FusedGraphIR]:

@@ -12,8 +12,8 @@ module provides the same shape of result from plain ``torch.fx``:
 3. grouping: every call node gets a *stage* = number of kernel boundaries on the longest path that
    reaches it.  A boundary is an edge that cannot stay inside one fused kernel: out of a ``Reducer`` or
    an aggregating ``sum``, into a ``Selector`` (a gather needs the whole source tensor), between values
-   of different leading dimension, and from/to an in-place write of a model tensor that is also read
-   elsewhere.  Nodes of equal stage joined by non-boundary edges form one fused sub-module; pure
+   of different leading dimension, and between an in-place write of a model tensor and a gather of the
+   same tensor (per-item reads and writes of one tensor may share a kernel).  Nodes of equal stage joined by non-boundary edges form one fused sub-module; pure
    element-wise groups of equal stage and equal length are merged into one;
 4. a top-level graph that calls the fused sub-modules in stage order.
 """
@@ -137,6 +137,14 @@ def group_nodes(gm: fx.GraphModule) -> List[List[fx.Node]]:
     deps: Dict[fx.Node, List[Tuple[fx.Node, bool]]] = {n: [] for n in calls}
     last_writer: Dict[str, fx.Node] = {}
     readers: Dict[str, List[fx.Node]] = {}
+    # A model tensor that is stored to and read by per-item operations of the same length can stay in one
+    # kernel: the item is loaded once, ``x[:] = v`` and ``x.add_(v)`` also update the register copy, and
+    # later operations of the kernel see the new value (the reference generates exactly that,
+    # codegen/merged_gen_core.py:203-213).  ``copy_`` does not refresh the register, and a gather needs the
+    # whole tensor as it is before or after the store, never in between: those cross a kernel boundary.
+    def refreshes_register(w: fx.Node) -> bool:
+        return w.target is operator.setitem or w.target == "add_"
+
     for n in calls:
         written = _is_write(n)
         for p in n.all_input_nodes:
@@ -145,14 +153,15 @@ def group_nodes(gm: fx.GraphModule) -> List[List[fx.Node]]:
                 if p is written:
                     for r in readers.get(key, []):
                         if r is not n:
-                            deps[n].append((r, True))      # write after read
+                            deps[n].append((r, kind[r] == "selector"))      # write after read
                     if key in last_writer:
-                        deps[n].append((last_writer[key], True))
+                        deps[n].append((last_writer[key], not refreshes_register(last_writer[key])))
                     last_writer[key] = n
                     readers[key] = []
                 else:
-                    if key in last_writer:
-                        deps[n].append((last_writer[key], True))   # read after write
+                    if key in last_writer:                                   # read after write
+                        w = last_writer[key]
+                        deps[n].append((w, kind[n] == "selector" or not refreshes_register(w)))
                     readers.setdefault(key, []).append(n)
                 continue
             if p not in deps:

@@ -160,7 +160,8 @@ def test_broadcast_along_the_edge_dimension_is_rejected_not_generated():
     assert torch.allclose(compiled.out.sum(), torch.tensor(1.0))
 
 
-@pytest.mark.parametrize("name,steps,tol", [("system", 2, 1e-14), ("spring", 3, 2e-5), ("swe", 2, 1e-12)])
+@pytest.mark.parametrize("name,steps,tol", [("system", 2, 1e-14), ("spring", 3, 2e-5), ("swe", 2, 1e-12),
+                                            ("swe_parts", 1, 0), ("swe_init", 1, 1e-13)])
 def test_replaced_model_matches_original_through_the_wrapper(name, steps, tol):
     eager, traced = MODELS[name](), MODELS[name]()
     [compiled] = esr.compile([traced], "torch")
@@ -237,6 +238,26 @@ def test_edge_ordering_helpers():
     assert pairs == {(0, 1), (1, 2), (2, 0), (1, 0), (2, 1), (0, 2)}
     assert torch.equal(w3, torch.tensor([10.0, 20.0, 30.0])[origin])
     assert all((sg > 0) == ((int(s), int(d)) in {(0, 1), (1, 2), (2, 0)}) for s, d, sg in zip(s2, d2, sign))
+
+
+def test_assembled_geometry_is_closed_and_feeds_the_model():
+    from flexspmv_amd.drivers.shallow_water_assembly import assemble, mesh_for_model
+    mesh, parts, init = assemble(400)
+    nc = mesh["cells"].shape[0]
+    # the collected ids are the cells' point ids seen from each face
+    assert torch.equal(torch.stack([p.data for p in parts.src_p], 1), mesh["cells"][mesh["src"]])
+    assert torch.equal(torch.stack([p.data for p in parts.bp], 1), mesh["bpoints"])
+    # every cell's inward face normals (interior + wall) close the polygon; areas tile the unit square
+    for a, b in ((init.sx, init.bsx), (init.sy, init.bsy)):
+        closed = torch.zeros(nc, dtype=torch.float64).index_add_(0, mesh["dst"], a.data).index_add_(0, mesh["bcells"], b.data)
+        assert float(closed.abs().max()) < 1e-14
+    assert abs(float(init.area.sum()) - 1.0) < 1e-13
+    assert 0.0 < float(init.alpha.min()) and float(init.alpha.max()) < 1.0
+    model = ShallowWaterEquation(mesh_for_model(mesh, init), dt=0.002)
+    mass = float((model.h * model.area).sum())
+    for _ in range(20):
+        model()
+    assert abs(float((model.h * model.area).sum()) - mass) < 1e-13 and float(model.h.max()) < 1.2
 
 
 def test_swe_conserves_mass():
