@@ -44,14 +44,17 @@ template <typename V, int N> __device__ __forceinline__ void zero(Pack<V, N>& a)
   for (int i = 0; i < N; ++i) a.v[i] = V(0);
 }
 
-// Streaming (read-once) loads and write-once stores bypass temporal caching so that gathered vertex
-// data, not the edge stream, occupies L2.
-#ifdef FLEX_TUNE_PLAIN_STREAMS  // tuning switch: ordinary (temporal) loads and stores for the streams
-template <typename T> __device__ __forceinline__ T stream_load(const T* p) { return *p; }
-template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) { *p = v; }
-#else
+// Loads of the read-once edge streams and stores of the write-once outputs.  Two tuning switches mark
+// them non-temporal; plain accesses measured faster for both on MI355X.
+#ifdef FLEX_TUNE_NT_LOADS
 template <typename T> __device__ __forceinline__ T stream_load(const T* p) { return __builtin_nontemporal_load(p); }
+#else
+template <typename T> __device__ __forceinline__ T stream_load(const T* p) { return *p; }
+#endif
+#ifdef FLEX_TUNE_NT_STORES
 template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) { __builtin_nontemporal_store(v, p); }
+#else
+template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) { *p = v; }
 #endif
 
 // Merge-path coordinate on diagonal `diag` of the merge of A = row_end[0..num_rows) (end offset of each
@@ -99,9 +102,8 @@ __device__ __forceinline__ int2 merge_path_search_interp(int diag, const int* __
 // One search per tile boundary: coords[t] is where tile t starts, coords[num_tiles] where the path ends.
 __global__ void __launch_bounds__(256)
 tile_search_kernel(int num_tiles, int tile_items, const int* __restrict__ row_end, int num_rows, int nnz,
-                   int2* __restrict__ coords, unsigned* __restrict__ ticket) {
+                   int2* __restrict__ coords) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t == 0) *ticket = 0u;  // arms fixup_kernel's last-block detection
   if (t > num_tiles) return;
   const long long d = (long long)t * tile_items;
   const int diag = (int)min(d, (long long)num_rows + nnz);
@@ -112,24 +114,22 @@ tile_search_kernel(int num_tiles, int tile_items, const int* __restrict__ row_en
 #endif
 }
 
-// Which tile a block works on.  By default tile = block: neighbouring tiles run at the same time on
-// different XCDs, which measured fastest on the stencil and mesh workloads.  The tuning switch
-// FLEX_TUNE_XCD_CHUNKS instead gives each XCD (block % 8) a contiguous range of tiles.
-__device__ __forceinline__ int tile_of_block(int block, int num_tiles) {
-#ifdef FLEX_TUNE_XCD_CHUNKS
-  const int per = (num_tiles + NUM_XCD - 1) / NUM_XCD;
-  return (block % NUM_XCD) * per + block / NUM_XCD;
-#else
-  (void)num_tiles;
-  return block;
+// Which tile a block works on.  Blocks are dealt to the 8 XCDs round-robin (block % 8), each XCD with
+// its own L2.  XCD_RUN consecutive tiles go to the same XCD, so that neighbouring tiles - which gather
+// overlapping vertex data - share an L2, while all XCDs still work inside one window of 8 * XCD_RUN tiles.
+#ifndef FLEX_TUNE_XCD_RUN
+#define FLEX_TUNE_XCD_RUN 1
 #endif
+constexpr int XCD_RUN = FLEX_TUNE_XCD_RUN;
+__device__ __forceinline__ int tile_of_block(int block, int num_tiles) {
+  (void)num_tiles;
+  if constexpr (XCD_RUN == 1) return block;
+  const int xcd = block % NUM_XCD, seq = block / NUM_XCD;
+  return ((seq / XCD_RUN) * NUM_XCD + xcd) * XCD_RUN + seq % XCD_RUN;
 }
 inline int grid_for_tiles(int num_tiles) {
-#ifdef FLEX_TUNE_XCD_CHUNKS
-  return (num_tiles + NUM_XCD - 1) / NUM_XCD * NUM_XCD;
-#else
-  return num_tiles;
-#endif
+  constexpr int WINDOW = NUM_XCD * XCD_RUN;
+  return XCD_RUN == 1 ? num_tiles : (num_tiles + WINDOW - 1) / WINDOW * WINDOW;
 }
 
 // ----------------------------------------------------------------------------------------------
@@ -303,7 +303,12 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
       };
 #pragma unroll
       for (int it = 0; it < ROW_PATH_UNROLL; ++it) {
-        if (it < len) add_edge(start + it, xv[it]);
+        if (it < len) {
+#ifdef FLEX_TUNE_ROW_BRANCH  // tuning switch: keep the predicate as a branch on the exec mask instead of selects
+          asm volatile("" ::: "memory");
+#endif
+          add_edge(start + it, xv[it]);
+        }
       }
       for (int it = ROW_PATH_UNROLL; it < len; ++it) {
         Pack<V, XCH> x;
@@ -553,18 +558,19 @@ flat_kernel(const typename G::Params p, const int nnz, const int num_tiles,
 }
 
 // ----------------------------------------------------------------------------------------------
-// Fix-up: fold tile carries into their rows (tile order) and finish the aggregators.
+// Fix-up: fold tile carries into their rows (tile order) and pre-reduce the aggregator partials.
 // Block b handles tiles [b*BLOCK, (b+1)*BLOCK): a thread owns the carry of one tile and, when it is
 // the first tile of a run that carries into the same row, adds the whole run to that row.  The
 // block's aggregator partials (PARTS_PER_TILE per tile, one per wavefront of the reducer block) are
-// summed in a fixed order into block_partials[b]; the block that finishes last adds the blocks'
-// partials, again in a fixed order, and assigns the outputs (no floating-point atomics anywhere).
+// summed in a fixed order into block_partials[b]; aggregate_kernel adds those, again in a fixed order.
+// (Finishing the sum in the last fix-up block to finish, found with a ticket counter, was measured and
+// is slower: the release fence each block needs writes the XCD's whole L2 back, output rows included.)
 // ----------------------------------------------------------------------------------------------
 template <class G, int BLOCK, int PARTS_PER_TILE>
 __global__ void __launch_bounds__(BLOCK)
 fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restrict__ carry_row,
              const typename G::Value* __restrict__ carry_val, const typename G::Value* __restrict__ agg_partials,
-             typename G::Value* __restrict__ block_partials, unsigned* __restrict__ ticket) {
+             typename G::Value* __restrict__ block_partials) {
   using V = typename G::Value;
   constexpr int RED = G::RED_WIDTH, AGG = G::AGG_WIDTH;
   constexpr int NW = BLOCK / WAVE;
@@ -601,49 +607,12 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
       for (int c = 0; c < AGG; ++c) s_wave_agg[threadIdx.x / WAVE][c] = acc.v[c];
     }
     __syncthreads();
-    __shared__ bool s_is_last;
     if (threadIdx.x == 0) {
 #pragma unroll
       for (int c = 0; c < AGG; ++c) {
         V s = s_wave_agg[0][c];
         for (int w = 1; w < NW; ++w) s += s_wave_agg[w][c];
-        __hip_atomic_store(&block_partials[(size_t)blockIdx.x * AGG + c], s, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-      }
-      // The block that draws the last ticket sees every other block's partial: each block publishes
-      // its partial before taking a ticket (release), the last block acquires after taking its own.
-      __atomic_thread_fence(__ATOMIC_RELEASE);
-      const unsigned drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-      s_is_last = (drawn == gridDim.x - 1);
-    }
-    __syncthreads();
-    if (s_is_last) {
-      __atomic_thread_fence(__ATOMIC_ACQUIRE);
-      // ordered final sum over the blocks' partials (same order on every run)
-      Pack<V, AGG> fin;
-      zero(fin);
-      for (int j = threadIdx.x; j < (int)gridDim.x; j += BLOCK) {
-#pragma unroll
-        for (int c = 0; c < AGG; ++c)
-          fin.v[c] += __hip_atomic_load(&block_partials[(size_t)j * AGG + c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      wave_sum_to_last_lane<V, AGG>(fin.v);
-      __syncthreads();  // s_wave_agg is reused
-      if ((threadIdx.x & (WAVE - 1)) == WAVE - 1) {
-#pragma unroll
-        for (int c = 0; c < AGG; ++c) s_wave_agg[threadIdx.x / WAVE][c] = fin.v[c];
-      }
-      __syncthreads();
-      if (threadIdx.x == 0) {
-        Pack<V, AGG> total;
-#pragma unroll
-        for (int c = 0; c < AGG; ++c) {
-          V s = s_wave_agg[0][c];
-          for (int w = 1; w < NW; ++w) s += s_wave_agg[w][c];
-          total.v[c] = s;
-        }
-        G::store_agg(p, total);
-        *ticket = 0u;  // re-armed for launches that reuse the tile table and skip the search kernel
+        block_partials[(size_t)blockIdx.x * AGG + c] = s;
       }
     }
   }

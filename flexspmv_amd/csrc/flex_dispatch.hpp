@@ -83,7 +83,7 @@ struct Dispatch {
     int num_tiles;
     int flat_blocks;
     int carry_blocks;
-    size_t off_coords, off_ticket, off_carry_row, off_carry_val, off_partials, off_block_partials, total;
+    size_t off_coords, off_carry_row, off_carry_val, off_partials, off_block_partials, total;
   };
 
   static bool layout(int64_t num_rows, int64_t ne, Layout& l) {
@@ -94,8 +94,6 @@ struct Dispatch {
     size_t off = 0;
     l.off_coords = off;
     if (REDUCER) off += align_up(sizeof(int2) * ((size_t)l.num_tiles + 1));
-    l.off_ticket = off;
-    if (REDUCER) off += align_up(sizeof(unsigned));
     l.off_carry_row = off;
     if (REDUCER) off += align_up(sizeof(int) * (size_t)l.num_tiles);
     l.off_carry_val = off;
@@ -142,11 +140,10 @@ struct Dispatch {
       int* carry_row = (int*)(ws + l.off_carry_row);
       V* carry_val = (V*)(ws + l.off_carry_val);
 
-      unsigned* ticket = (unsigned*)(ws + l.off_ticket);
       if ((a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0) {
         const int search_blocks = (l.num_tiles + 1 + 255) / 256;
         hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(256), 0, stream, l.num_tiles, TILE,
-                           row_end, num_rows, nnz, coords, ticket);
+                           row_end, num_rows, nnz, coords);
       }
       if (timed) (void)hipEventRecord(g_timer.start, stream);
       hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid_for_tiles(l.num_tiles)), dim3(BLOCK), 0, stream,
@@ -154,8 +151,11 @@ struct Dispatch {
       if (timed) g_timer.armed = (hipEventRecord(g_timer.stop, stream) == hipSuccess);
       V* block_partials = (V*)(ws + l.off_block_partials);
       hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, BLOCK / WAVE>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0, stream, p,
-                         l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials, block_partials,
-                         ticket);
+                         l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials, block_partials);
+      if (G::AGG_WIDTH > 0) {
+        hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
+                           (const V*)block_partials, l.carry_blocks);
+      }
     } else {
       int grid = resident_grid(flat_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
       if (grid > l.num_tiles) grid = l.num_tiles;
