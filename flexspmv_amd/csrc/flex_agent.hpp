@@ -170,7 +170,10 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
   constexpr int XCHN = XCH > 0 ? XCH : 1;
   constexpr int OUT_CAP = 2 * BLOCK;          // merge path: finished rows of a tile buffered in LDS
   constexpr int OUT_STRIDE = OUT_CAP + WAVE;  // + one dump slot per lane for items that close no row
-  constexpr int ROW_PATH_MAX_LEN = 32;        // longest row the row path accepts
+#ifndef FLEX_TUNE_ROW_PATH_MAX_LEN
+#define FLEX_TUNE_ROW_PATH_MAX_LEN 32
+#endif
+  constexpr int ROW_PATH_MAX_LEN = FLEX_TUNE_ROW_PATH_MAX_LEN;  // longest row the row path accepts (0: never)
   constexpr int ROW_PATH_UNROLL = 8;          // non-zeros of a row read from LDS up front
   constexpr int ROW_PATH_MAX_ROWS = BLOCK + WAVE;  // rows (incl. the open one) whose ends are prefetched
   static_assert((IPT & (IPT - 1)) == 0 && IPT <= 32, "a thread's items must sit inside one bitmap word");
@@ -270,14 +273,28 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
       }
     }
   }
-  const bool my_vote = (max(len1, len2) > ROW_PATH_MAX_LEN) | !few_rows;
-  if (lane == 0) s_vote[wave] = (__builtin_amdgcn_ballot_w64(my_vote) != 0ull) ? 1 : 0;
-  else (void)__builtin_amdgcn_ballot_w64(my_vote);
+  // ... and are the rows regular?  A thread per row pays for the longest row of its wavefront, so the row
+  // path only wins when no row is much longer than the tile's average (meshes, stencils); on skewed
+  // tiles with short rows the merge path measured about 10 % faster.
+  const int longest = max(len1, len2);
+#ifdef FLEX_TUNE_ROW_PATH_ANY_SHAPE  // tuning switch: length limit only
+  const bool uneven = false;
+#else
+  const bool uneven = 4 * (longest - 1) * (R + 1) > 5 * Z;  // longer than 1.25 x average + 1
+#endif
+  const bool my_vote = (longest > ROW_PATH_MAX_LEN) | !few_rows | uneven;
+  // the ballot is taken by the whole wavefront (inside a branch it would only see the branch's lanes)
+  const unsigned long long wave_votes = __builtin_amdgcn_ballot_w64(my_vote);
+  if (lane == 0) s_vote[wave] = (wave_votes != 0ull) ? 1 : 0;
   __syncthreads();
   int any_vote = 0;
 #pragma unroll
   for (int w = 0; w < NW; ++w) any_vote |= s_vote[w];
+#ifdef FLEX_TUNE_FORCE_MERGE  // tuning switch: always the merge path, decided at run time (same code)
+  const bool irregular = any_vote != 0 || num_tiles > 0;
+#else
   const bool irregular = any_vote != 0;
+#endif
 
   if (!irregular) {
     // ---------------- ROW path ----------------
