@@ -214,6 +214,17 @@ def _emit_map(op: Dict[str, Any], vars: Dict[str, Var], edge: str) -> List[str]:
     a = [_arg(x) for x in op["args"]] if o not in ("getitem", "setitem") else None
     T = f"TensorOutput_{name}_T"
     binary = {"add": "+", "sub": "-", "mul": "*", "pow": "^", "truediv": "/", "lt": "<", "gt": ">"}
+    if o == "pow" and isinstance(op["args"][1], (int, float)) and not isinstance(op["args"][1], bool) \
+            and isinstance(arg_name(op["args"][0]), str):
+        # literal exponents 0.5 and 1..4 take the direct form (same value to within an ulp of pow)
+        e = op["args"][1]
+        base = vars.get(a[0])
+        scalar = base is not None and base.kind == "scalar"
+        if e == 0.5:
+            return [f"{T} {name}(flex::v_sqrt({a[0]}));" if scalar else f"{T} {name} = {a[0]}.sqrt();"]
+        if float(e).is_integer() and 1 <= int(e) <= 4:
+            return [f"{T} {name}(flex::v_ipow<{int(e)}>({a[0]}));" if scalar
+                    else f"{T} {name} = {a[0]}.template ipow<{int(e)}>();"]
     if o in binary:
         return [f"{T} {name} = {a[0]} {binary[o]} {a[1]};"]
     if o == "neg":

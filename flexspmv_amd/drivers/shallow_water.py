@@ -14,6 +14,7 @@ import numpy as np
 import torch
 
 from .. import frontend as esr
+from ..python_wrapper.edge_order import morton_order
 
 
 def synthetic_mesh(points: int = 2000, seed: int = 3, dtype=torch.float64, device="cpu") -> Dict[str, torch.Tensor]:
@@ -30,6 +31,11 @@ def synthetic_mesh(points: int = 2000, seed: int = 3, dtype=torch.float64, devic
     tri = Delaunay(pts)
     cells, nbr = tri.simplices, tri.neighbors           # nbr[c, k]: cell opposite vertex k (-1: wall)
     nc = len(cells)
+    order_c = morton_order(pts[cells].mean(axis=1))     # number the cells with spatial locality
+    new_id = np.empty(nc, dtype=np.int64)
+    new_id[order_c] = np.arange(nc)
+    cells, nbr = cells[order_c], nbr[order_c]
+    nbr = np.where(nbr >= 0, new_id[np.maximum(nbr, 0)], -1)
     centroid = pts[cells].mean(axis=1)
     p0, p1, p2 = pts[cells[:, 0]], pts[cells[:, 1]], pts[cells[:, 2]]
     area = 0.5 * np.abs((p1[:, 0] - p0[:, 0]) * (p2[:, 1] - p0[:, 1]) - (p2[:, 0] - p0[:, 0]) * (p1[:, 1] - p0[:, 1]))

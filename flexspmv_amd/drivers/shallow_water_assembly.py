@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 from .. import frontend as esr
+from ..python_wrapper.edge_order import morton_order
 
 
 def synthetic_topology(points: int = 900, seed: int = 3, device="cpu") -> Dict[str, torch.Tensor]:
@@ -30,6 +31,11 @@ def synthetic_topology(points: int = 900, seed: int = 3, device="cpu") -> Dict[s
     pts = (np.stack([gx.ravel(), gy.ravel()], axis=1) + jitter) / (m - 1) - 0.5
     tri = Delaunay(pts)
     cells, nbr = tri.simplices.astype(np.int64), tri.neighbors
+    order_c = morton_order(pts[cells].mean(axis=1))     # number the cells with spatial locality
+    new_id = np.empty(len(cells), dtype=np.int64)
+    new_id[order_c] = np.arange(len(cells))
+    cells, nbr = cells[order_c], nbr[order_c]
+    nbr = np.where(nbr >= 0, new_id[np.maximum(nbr, 0)], -1)
     dst, k = np.nonzero(nbr >= 0)
     src = nbr[dst, k]
     order = np.lexsort((src, dst))

@@ -181,6 +181,16 @@ def shallow_water_mesh(points: int = 1_000_000, dtype="float64", seed: int = 3) 
     cells = tri.simplices                      # [C, 3]
     nbr = tri.neighbors                        # nbr[c, k] = cell opposite vertex k, -1 on the hull
     C = len(cells)
+    # Cells are numbered along a Morton curve through their centroids, as mesh generators and
+    # partitioners do: neighbouring cells get nearby numbers (the triangulation itself numbers them in
+    # an order without locality, which turns every gather into a random access).
+    from .python_wrapper.edge_order import morton_order
+    order_c = morton_order(pts[cells].mean(axis=1))
+    new_id = np.empty(C, dtype=np.int64)
+    new_id[order_c] = np.arange(C)
+    cells = cells[order_c]
+    nbr = nbr[order_c]
+    nbr = np.where(nbr >= 0, new_id[np.maximum(nbr, 0)], -1)
     cc, kk = np.nonzero(nbr >= 0)
     dst = cc.astype(np.int64)                  # the cell being updated
     src = nbr[cc, kk].astype(np.int64)
