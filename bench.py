@@ -173,6 +173,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="poisson3d", choices=sorted(DEFAULT_SIZE))
     ap.add_argument("--size", type=int, default=None, help="grid edge / R-MAT scale / point count")
+    ap.add_argument("--mtx", default=None, help="time SpMV on this MatrixMarket file instead of a generated workload "
+                                                "(float64 y = A x)")
+    ap.add_argument("--mtx-dot", action="store_true", help="with --mtx: the fused form y = A x and x . y")
     ap.add_argument("--all", action="store_true", help="also time the other four workloads (extra JSON key)")
     ap.add_argument("--cpu-runs", type=int, default=5, help="timed runs of the CPU baseline (0 = skip)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -191,7 +194,10 @@ def main() -> int:
     from flexspmv_amd import workloads as W
 
     size = a.size if a.size is not None else DEFAULT_SIZE[a.workload]
-    w = W.WORKLOADS[a.workload](size)
+    if a.mtx is not None:
+        w = W.matrix_market_spmv(a.mtx, fused_dot=a.mtx_dot)
+    else:
+        w = W.WORKLOADS[a.workload](size)
     head, head_outs = time_workload(w, a.steps, a.warmup)
     torch.cuda.empty_cache()
     if a.copy_calibration:
@@ -236,7 +242,9 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": DTYPE_TAG[head["dtype"]],
         "data": "synthetic",
-        "config": {"workload": f"{head['workload']} fused y=A*x and x.y ({head['graph']})", "ne": head["ne"],
+        "config": {"workload": f"{head['workload']} " + ("fused y=A*x and x.y" if head["graph"] == "spmv_dot"
+                                                        else "y=A*x" if head["graph"] == "csr_spmv" else "step")
+                               + f" ({head['graph']})", "ne": head["ne"],
                    "num_rows": head["num_rows"], "algorithmic_bytes": head["algorithmic_bytes"],
                    "policy": head["policy"]},
         "ms_per_step_trials": head["ms_per_step_trials"],
@@ -246,7 +254,8 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": head["kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["kernel_gbs"] / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(
-                         (a.workload, size, f"{head['policy']['block']}x{head['policy']['ipt'][head['dtype']]}")),
+                         (a.workload if a.mtx is None else "mtx", size,
+                          f"{head['policy']['block']}x{head['policy']['ipt'][head['dtype']]}")),
                      "kernel": "flex::reduce_kernel" if head["graph"] not in ("mass_sum", "map_store", "bpoints_copy")
                      else "flex::flat_kernel",
                      "kernel_ms": head["kernel_ms"]},

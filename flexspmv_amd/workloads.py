@@ -233,6 +233,40 @@ def mass_sum_of(swe: Workload) -> Workload:
                     algorithmic_bytes=2 * b * C + b, flops=2 * C, seed=swe.seed)
 
 
+def matrix_market_spmv(path: str, dtype="float64", seed: int = 7, fused_dot: bool = False) -> Workload:
+    """SpMV on a matrix read from a MatrixMarket file (the reference's CUDA harness takes one with
+    ``--mtx``, src/flex_spmv_full_red.cu:643): CSR with sorted columns, duplicate entries summed,
+    symmetric storage expanded; pattern matrices get unit values.  ``x`` is random in [-1, 1)."""
+    import os
+
+    import scipy.io
+    import scipy.sparse as sp
+    dtype = np.dtype(dtype)
+    a = sp.csr_matrix(scipy.io.mmread(path))
+    a.sum_duplicates()
+    a.sort_indices()
+    if a.nnz == 0:
+        raise ValueError(f"{path}: matrix has no entries")
+    if a.shape[0] + a.nnz >= 2 ** 31:
+        raise ValueError(f"{path}: rows + non-zeros do not fit 32-bit offsets")
+    rng = np.random.default_rng(seed)
+    x = rng.uniform(-1.0, 1.0, a.shape[1]).astype(dtype)
+    vals = np.ascontiguousarray(a.data.astype(dtype))
+    cols = np.ascontiguousarray(a.indices.astype(np.int32))
+    ptr = np.ascontiguousarray(a.indptr.astype(np.int32))
+    n, m, nnz, b = a.shape[0], a.shape[1], a.nnz, dtype.itemsize
+    name = "mtx_" + os.path.splitext(os.path.basename(path))[0]
+    if fused_dot:
+        if n != m:
+            raise ValueError("x . (A x) needs a square matrix")
+        rows = np.repeat(np.arange(n, dtype=np.int32), np.diff(ptr))
+        return Workload(name, "spmv_dot", {"vals": vals, "x": x, "selector_col_idx": cols, "selector_row_idx": rows},
+                        ptr, n, m, nnz, algorithmic_bytes=nnz * (4 + b) + 4 * (n + 1) + b * m + b * n + b,
+                        flops=2 * nnz + 2 * n, seed=seed, notes="selector_row_idx equals the row ids and is not read")
+    return Workload(name, "csr_spmv", {"vals": vals, "x": x, "selector_idx": cols}, ptr, n, m, nnz,
+                    algorithmic_bytes=nnz * (4 + b) + 4 * (n + 1) + b * m + b * n, flops=2 * nnz, seed=seed)
+
+
 WORKLOADS = {
     "laplacian2d": laplacian_2d_spmv,
     "spring_mass": spring_mass_grid,

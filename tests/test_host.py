@@ -4,6 +4,8 @@ import json
 import os
 import re
 
+import numpy as np
+
 import pytest
 
 from flexspmv_amd import build, graphs
@@ -171,3 +173,30 @@ def test_workspace_query():
     assert lib.flexspmv_workspace_bytes(1, 2**30, 2**30) == 0        # does not fit 32-bit offsets
     flat = _lib("bpoints_copy")
     assert flat.flexspmv_workspace_bytes(2, 100, 100) == 0           # map-only needs no scratch
+
+
+def test_matrix_market_workload(tmp_path):
+    """A MatrixMarket file becomes a CSR SpMV workload: symmetric storage expanded, duplicates summed,
+    columns sorted; the oracle's product equals scipy's."""
+    import scipy.io
+    import scipy.sparse as sp
+    from flexspmv_amd import graphs
+    from flexspmv_amd import workloads as W
+    from oracle.runner import run_oracle
+    rng = np.random.default_rng(0)
+    a = sp.random(40, 40, density=0.15, random_state=1, format="coo")
+    a = sp.coo_matrix(a + a.T)                              # symmetric: written in symmetric storage
+    path = str(tmp_path / "sym.mtx")
+    scipy.io.mmwrite(path, a, symmetry="symmetric")
+    w = W.matrix_market_spmv(path)
+    assert w.graph == "csr_spmv" and w.num_rows == 40 and w.ne == sp.csr_matrix(a).nnz
+    assert all(np.all(np.diff(w.tensors["selector_idx"][s:e]) > 0)
+               for s, e in zip(w.row_end_offsets[:-1], w.row_end_offsets[1:]))
+    (y,), _ = run_oracle(graphs.get("csr_spmv"), w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, 3)
+    assert np.allclose(y, sp.csr_matrix(a) @ w.tensors["x"], rtol=1e-13, atol=1e-15)
+    wd = W.matrix_market_spmv(path, fused_dot=True)
+    (y2, dot), _ = run_oracle(graphs.get("spmv_dot"), wd.tensors, wd.row_end_offsets, wd.num_rows, wd.num_cols, 3)
+    assert np.allclose(y2, y) and np.isclose(dot[0], wd.tensors["x"] @ y, rtol=1e-12)
+    with pytest.raises(ValueError):
+        scipy.io.mmwrite(str(tmp_path / "rect.mtx"), sp.random(5, 7, density=0.5, random_state=2))
+        W.matrix_market_spmv(str(tmp_path / "rect.mtx"), fused_dot=True)
