@@ -111,12 +111,24 @@ def main(argv=None) -> int:
     sync()
     t_replaced = (time.perf_counter() - t0) / a.steps
     worst, ok = compare_states(original_final, save_state(compiled), a.tolerance)
+    t_graph = None
+    if a.device.startswith("cuda") and all(v == "replaced" for v in report.values()):
+        from ..python_wrapper.graph_replay import capture_step
+        replay = capture_step(compiled)
+        replay()
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            replay()
+        sync()
+        t_graph = (time.perf_counter() - t0) / a.steps
     for k, v in report.items():
         print(f"  {k}: {v}")
     for k, v in worst.items():
         print(f"  {k}: max rel diff {v:.3e}")
     print(f"  ms per step: torch sub-modules {t_original * 1e3:.3f}, generated libraries {t_replaced * 1e3:.3f} "
-          f"({t_original / t_replaced:.2f}x)")
+          f"({t_original / t_replaced:.2f}x)"
+          + (f", the same replayed as one HIP graph {t_graph * 1e3:.3f} ({t_original / t_graph:.2f}x)" if t_graph else ""))
     print("PASSED" if ok else "FAILED")
     return 0 if ok else 1
 
