@@ -241,6 +241,49 @@ def test_rmat_scale_20_linearity_and_library_product():
     assert ((y1.double() - ref).abs() <= 1e-5 * ref.abs()).all()
 
 
+def test_shallow_water_1m_points_conservation_and_lake_at_rest():
+    """Full-size mesh (about 2 M cells, 6 M half-edges).  Every interior face appears once per direction
+    with opposite normals and the Rusanov flux is antisymmetric, so the fluxes summed over all cells cancel;
+    a lake at rest (constant depth, no momentum) has zero mass flux everywhere and, in cells without a wall
+    face, zero momentum flux (the scaled normals of a closed polygon add up to zero)."""
+    w = W.shallow_water_mesh(1_000_000)
+    ext = load_named(w.graph, build_if_missing=False)
+    names = ext.param_names()
+    args = W.launch_arguments(w, names, "cuda")
+    print(f"case swe 1M cells={w.num_rows} half-edges={w.ne}", flush=True)
+    fh, fu, fv = ext.merged_spmv_launch(*args)
+    for f in (fh, fu, fv):
+        scale = float(f.abs().sum())
+        assert abs(float(f.sum())) <= 1e-12 * scale
+    U = args[names.index("U")]
+    rest = torch.zeros_like(U)
+    rest[:, 0] = 1.25
+    args[names.index("U")] = rest
+    fh, fu, fv = ext.merged_spmv_launch(*args)
+    assert float(fh.abs().max()) == 0.0
+    ptr = args[names.index("row_end_offsets")].long()
+    interior = (ptr[1:] - ptr[:-1]) == 3                      # all three faces are interior faces
+    pressure_scale = 0.5 * 9.81 * 1.25 ** 2 * float(args[names.index("length")].max())
+    assert float(fu[interior].abs().max()) <= 1e-12 * pressure_scale
+    assert float(fv[interior].abs().max()) <= 1e-12 * pressure_scale
+    assert float(fu[~interior].abs().max()) > 0              # wall cells do feel the missing face
+
+
+def test_rmat_scale_22_against_the_library_product():
+    w = W.rmat_spmv(22)
+    ext = load_named(w.graph, build_if_missing=False)
+    names = ext.param_names()
+    args = W.launch_arguments(w, names, "cuda")
+    print(f"case rmat s22 rows={w.num_rows} nnz={w.ne}", flush=True)
+    (y,) = ext.merged_spmv_launch(*args)
+    A = torch.sparse_csr_tensor(args[names.index("row_end_offsets")].long(), args[names.index("selector_idx")].long(),
+                                args[names.index("vals")].double(), size=(w.num_rows, w.num_cols))
+    ref = (A @ args[names.index("x")].double().unsqueeze(1)).squeeze(1)
+    assert ((y.double() - ref).abs() <= 1e-5 * ref.abs()).all()      # all terms positive: the row scale is |ref|
+    empty = (torch.diff(args[names.index("row_end_offsets")]) == 0)
+    assert bool((y[empty] == 0).all())
+
+
 # ---------------------------------------------------------------------------------------------
 # error behaviour of the call surface (TORCH_CHECK -> RuntimeError in the reference)
 # ---------------------------------------------------------------------------------------------
