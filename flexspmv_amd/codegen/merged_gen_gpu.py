@@ -268,7 +268,8 @@ def _indent(lines: Sequence[str], n: int = 4) -> str:
 
 def _choose_ipt(kp: KernelPlan, value_bytes: int) -> int:
     """Items per thread so that one block's LDS stays inside LDS_BUDGET_BYTES."""
-    per_item = value_bytes * max(kp.xch_width, 1)
+    # LDS holds the per-edge exchange of a tile and, in the merge path, one finished total per row
+    per_item = value_bytes * max(kp.xch_width, kp.red_width, 1)
     for ipt in (8, 4, 2, 1):
         if BLOCK_THREADS * ipt * per_item <= LDS_BUDGET_BYTES:
             return ipt

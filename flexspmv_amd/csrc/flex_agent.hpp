@@ -168,7 +168,7 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
   constexpr int XCH = G::XCH_WIDTH, RED = G::RED_WIDTH, AGG = G::AGG_WIDTH, ROW = G::ROW_WIDTH;
   constexpr int REDN = RED > 0 ? RED : 1;
   constexpr int XCHN = XCH > 0 ? XCH : 1;
-  constexpr int OUT_CAP = 2 * BLOCK;          // merge path: finished rows of a tile buffered in LDS
+  constexpr int OUT_CAP = TILE;               // merge path: every row a tile can finish is buffered in LDS
   constexpr int OUT_STRIDE = OUT_CAP + WAVE;  // + one dump slot per lane for items that close no row
 #ifndef FLEX_TUNE_ROW_PATH_MAX_LEN
 #define FLEX_TUNE_ROW_PATH_MAX_LEN 32
@@ -376,7 +376,6 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
     const unsigned nzs = ~ends & (n_items >= IPT ? FULL : ((1u << n_items) - 1u));  // ... that are non-zeros
     const int xs = s_word_prefix[d0 >> 5] + __popc(word & ((1u << sh) - 1u));        // rows before my items
     const int ys = d0 - xs;                                                            // non-zeros before them
-    const bool direct = R > OUT_CAP;  // more rows than the LDS output buffer holds: store directly
 
     Pack<V, XCH> xv[IPT];
     int xrel[IPT];
@@ -423,12 +422,10 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
         }
       }
       // a row end parks the finished total in the output buffer (other items write a dump slot)
-      if (!direct) {
+      {
         const int slot = end ? xrel[it] : dump;
 #pragma unroll
         for (int c = 0; c < RED; ++c) s_out[c * OUT_STRIDE + slot] = tot.v[c];
-      } else if (end) {
-        G::store_row(p, x0 + xrel[it], tot);
       }
 #pragma unroll
       for (int c = 0; c < RED; ++c) tot.v[c] = end ? V(0) : tot.v[c];
@@ -477,15 +474,8 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
     // the first row a thread closed may have started in earlier threads: add what they carried in
     // (only this thread ever touches that row's slot, so a plain read-modify-write is safe)
     if (ends != 0u && in_key == xs) {
-      if (!direct) {
 #pragma unroll
-        for (int c = 0; c < RED; ++c) s_out[c * OUT_STRIDE + xs] += in_val[c];
-      } else {
-        Pack<V, RED> cin;
-#pragma unroll
-        for (int c = 0; c < RED; ++c) cin.v[c] = in_val[c];
-        G::add_row(p, x0 + xs, cin);
-      }
+      for (int c = 0; c < RED; ++c) s_out[c * OUT_STRIDE + xs] += in_val[c];
     }
     // tile carry-out: what the tile accumulated for the row still open at its end
     if (tid == BLOCK - 1) {
@@ -501,13 +491,11 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
     __syncthreads();
 
     // the tile's finished rows leave LDS as coalesced stores
-    if (!direct) {
-      for (int i = tid; i < R; i += BLOCK) {
-        Pack<V, RED> t;
+    for (int i = tid; i < R; i += BLOCK) {
+      Pack<V, RED> t;
 #pragma unroll
-        for (int c = 0; c < RED; ++c) t.v[c] = s_out[c * OUT_STRIDE + i];
-        G::store_row(p, x0 + i, t);
-      }
+      for (int c = 0; c < RED; ++c) t.v[c] = s_out[c * OUT_STRIDE + i];
+      G::store_row(p, x0 + i, t);
     }
   }
 
