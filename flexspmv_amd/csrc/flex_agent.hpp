@@ -5,8 +5,9 @@
 //   G::Params                      pointer bundle (kernel argument)
 //   XCH / RED / AGG / ROW widths   number of V values per edge passed through LDS, per-row reduced,
 //                                  globally summed, and staged per tile row
-//   stage1(p, e, xch, agg)         selector + map for edge e in coalesced order; fills xch, adds to agg
-//   stage2(p, e, row, xch, rv, tot, agg)   the part of the map that needs the row; adds to tot / agg
+//   fetch / gather                 first-level (streamed) and second-level (gathered) loads of edge e
+//   stage1(p, e, f, g, xch, agg)   the map for edge e in coalesced order; fills xch, adds to agg
+//   contrib(p, e, row, xch, rv, tot, agg)  the part of the map that needs the row; assigns tot / agg
 //   load_row / store_row / add_row / store_agg   row-aligned sources and outputs
 //
 // What the kernels replace in the reference (CUDA + CUB):
@@ -23,8 +24,9 @@
 //     fixup_kernel folds in tile order (same result on every run);
 //   * aggregators are block partials + one ordered final sum instead of floating-point atomics;
 //   * a reducer and an aggregator can share one pass over the edges;
-//   * blocks are mapped to tiles so that each XCD (one L2 each, workgroups are dealt round-robin to the
-//     8 XCDs) walks a contiguous range of tiles and gathered vertex data stays in that XCD's L2.
+//   * one small independent block per tile; block b takes tile b, so the 8 XCDs (one L2 each, workgroups
+//     are dealt to them round-robin) work side by side on neighbouring tiles.  Longer runs of tiles per
+//     XCD cut the re-fetching of gathered data but measured no faster (tuning switch FLEX_TUNE_XCD_RUN).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
