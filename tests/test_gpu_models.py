@@ -138,3 +138,17 @@ def test_graph_replay_of_a_model_step_matches_eager_launches():
     for k in want:
         assert torch.equal(want[k], got[k]), k
     assert float(scratch[0]) == steps
+
+
+def test_conjugate_gradients_on_the_fused_poisson_operator():
+    """The solver loop around the fused ``A p`` / ``p . A p`` launch converges to the solution of a
+    manufactured problem, and launches after the first reuse the tile table."""
+    from flexspmv_amd.drivers.poisson_cg import conjugate_gradients, fused_operator
+    print("case poisson cg 48^3", flush=True)
+    apply, n = fused_operator(48)
+    truth = torch.rand(n, dtype=torch.float64, device="cuda", generator=torch.Generator("cuda").manual_seed(1))
+    b, _ = apply(truth.clone())
+    b = b.clone()
+    x, iterations, residual = conjugate_gradients(apply, b, tol=1e-10, maxiter=2000)
+    assert residual <= 1e-10 and iterations < 400
+    assert float((x - truth).abs().max()) <= 1e-8
