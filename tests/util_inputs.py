@@ -18,7 +18,7 @@ def row_structure(kind, rng, tile=2048):
         lens[2000] = tile
     elif kind == "one_long_row":  # a single row far longer than a tile: every tile carries into it
         lens = np.array([0, 0, 9 * tile + 5, 0])
-    elif kind == "mostly_empty":  # > 512 row ends in a tile: merge path with direct stores
+    elif kind == "mostly_empty":  # many row ends per tile: merge path, every row through the LDS buffer
         lens = (rng.random(20000) < 0.05).astype(np.int64) * rng.integers(1, 40, 20000)
         lens[-1] = 7
     elif kind == "tiny":
@@ -28,6 +28,14 @@ def row_structure(kind, rng, tile=2048):
     elif kind == "len33":         # one row just over the row-path limit inside regular rows
         lens = np.full(900, 5)
         lens[450] = 33
+    elif kind == "empty_tiles":   # tiles that consist of row ends only (R = tile), between ordinary rows
+        lens = np.concatenate([np.full(300, 6), np.zeros(3 * tile + 100, dtype=np.int64), np.full(300, 9)])
+    elif kind == "uniform_30":    # row path, rows longer than its unrolled part
+        lens = np.full(700, 30)
+    elif kind == "uneven_short":  # all rows short but of very different lengths: merge path by the evenness rule
+        lens = rng.integers(1, 31, 3000)
+    elif kind == "rows_5":        # more rows per tile than the row path prefetches: merge path on a regular matrix
+        lens = np.full(4000, 4) + (np.arange(4000) % 2)
     else:
         raise ValueError(kind)
     if lens.sum() == 0:
@@ -35,7 +43,8 @@ def row_structure(kind, rng, tile=2048):
     return np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
 
 
-STRUCTURES = ["mesh", "mesh_with_gaps", "skewed", "one_long_row", "mostly_empty", "tiny", "exact_tiles", "len33"]
+STRUCTURES = ["mesh", "mesh_with_gaps", "skewed", "one_long_row", "mostly_empty", "tiny", "exact_tiles", "len33",
+              "empty_tiles", "uniform_30", "uneven_short", "rows_5"]
 
 
 def make_inputs(ir, dtype, rng, row_ptr=None, ne=None, positive=True):
