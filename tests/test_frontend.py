@@ -282,3 +282,17 @@ def test_spring_energy_is_half_k_stretch_squared():
     assert abs(float(m.energy) - expected) < 1e-12 * expected
     # internal forces cancel
     assert float(m.force.sum(dim=0).abs().max()) < 1e-12
+
+
+def test_reference_named_entry_point_writes_the_hip_source(tmp_path):
+    """``generate_cuda_code_from_graph(submodule, traced_model)`` - the call the reference's drivers make
+    (easier_spmv.py:157) - traces the fused sub-module and writes its translation unit."""
+    from flexspmv_amd.codegen.merged_gen_gpu import generate_cuda_code_from_graph
+    from flexspmv_amd.python_wrapper.accelerate import get_submodules
+    [compiled] = esr.compile([make_system()], "torch")
+    submodules, nodes = get_submodules(compiled)
+    path, signature = generate_cuda_code_from_graph(submodules[0], compiled, out_dir=str(tmp_path))
+    text = open(path).read()
+    assert path.endswith(".hip") and "flexspmv_launch" in text and "struct Graph" in text
+    assert [p["name"] for p in signature["params"]][-3:] == ["row_end_offsets", "num_rows", "num_cols"]
+    assert signature["index_inputs"] == ["selector_1_idx", "selector_2_idx"]
