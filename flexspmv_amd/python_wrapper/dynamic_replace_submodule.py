@@ -13,7 +13,10 @@ Deliberate differences:
   the reference walks ``named_modules()`` and stops at the first Reducer
   (dynamic_replace_submodule.py:65-72), which drops selectors registered after it;
 * the reducer's row ids must be sorted for the COO -> CSR conversion to describe them
-  (dynamic_replace_submodule.py:20-41 assumes it); unsorted ids raise instead of giving a wrong sum;
+  (dynamic_replace_submodule.py:20-41 assumes it, and the reference's own toy model draws them unsorted,
+  easier_spmv.py:126-127).  ``_coo_rows_to_csr_ptr`` raises on unsorted ids; ``build_wrapper`` handles them:
+  it sorts the edges by row once (stable, on the ids' device), permutes the selector index buffers once,
+  and per call permutes the streamed edge tensors in and the per-edge results back out;
 * outputs are returned in the shapes the fused sub-module itself produces (``[n, 2, 1]`` stays that way).
 """
 from __future__ import annotations
@@ -104,6 +107,20 @@ def _written_inputs(gm) -> List[str]:
     return out
 
 
+def _per_edge_outputs(gm) -> List[bool]:
+    """For every returned value: is it a per-edge map result (as opposed to a reducer or an aggregate)?"""
+    for node in gm.graph.nodes:
+        if node.op == "output":
+            returned = node.args[0] if isinstance(node.args[0], (list, tuple)) else [node.args[0]]
+            flags = []
+            for r in returned:
+                reduction = (r.op == "call_module" and type(gm.get_submodule(r.target)) is Reducer) or \
+                            (r.op == "call_function" and getattr(r.target, "__name__", "") == "sum")
+                flags.append(not reduction)
+            return flags
+    return []
+
+
 def _output_shapes(gm) -> List[Tuple[int, ...]]:
     for node in gm.graph.nodes:
         if node.op == "output":
@@ -118,7 +135,8 @@ class _DynamicCudaWrapper(nn.Module):
     def __init__(self, ext_module, input_param_names: List[str], non_gather_value_inputs: List[str],
                  gather_value_inputs: List[str], selector_idx_tensors: List[torch.Tensor],
                  row_end_offsets: Optional[torch.Tensor], output_shapes: Optional[List[Tuple[int, ...]]] = None,
-                 written_inputs: Iterable[str] = ()) -> None:
+                 written_inputs: Iterable[str] = (), edge_permutation: Optional[torch.Tensor] = None,
+                 per_edge_outputs: Optional[List[bool]] = None) -> None:
         super().__init__()
         names: List[str] = []
         for i, t in enumerate(selector_idx_tensors):
@@ -135,6 +153,10 @@ class _DynamicCudaWrapper(nn.Module):
                     raise RuntimeError("row_end_offsets does not fit 32-bit offsets")
                 reo = reo.to(torch.int32)
         self.register_buffer("row_end_offsets", reo, persistent=False)
+        # edges sorted by row when the model's edge list is not: position k of the kernel's edge order
+        # holds the model's edge edge_permutation[k]
+        self.register_buffer("edge_permutation", edge_permutation, persistent=False)
+        self._per_edge_outputs = list(per_edge_outputs) if per_edge_outputs is not None else None
         self._ext = ext_module
         self._input_param_names = list(input_param_names)
         self._non_gather_value_inputs = list(non_gather_value_inputs)
@@ -174,15 +196,27 @@ class _DynamicCudaWrapper(nn.Module):
         if num_rows is None:
             num_rows = num_cols
 
+        perm = None
+        if self.edge_permutation is not None:
+            perm = self._on("edge_permutation", device)
+            for n in self._non_gather_value_inputs:
+                arg_map[n] = arg_map[n].index_select(0, perm)
         call_args = [arg_map[n] for n in self._non_gather_value_inputs]
         call_args += [arg_map[n] for n in self._gather_value_inputs]
         call_args += [self._on(b, device) for b in self._selector_buf_names]
         call_args += [ro, num_rows, num_cols]
 
         outs = self._ext.merged_spmv_launch(*call_args)
+        if perm is not None:            # per-edge stores went to the sorted copies: put them back
+            for n, a in zip(self._input_param_names, args):
+                if n in self._written_inputs and n in self._non_gather_value_inputs:
+                    a.index_copy_(0, perm, arg_map[n].view((a.shape[0],) + tuple(a.shape[1:])))
         if outs is None:
             return []
         outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
+        if perm is not None and self._per_edge_outputs is not None:
+            outs = [torch.empty_like(o).index_copy_(0, perm, o) if per_edge else o
+                    for o, per_edge in zip(outs, self._per_edge_outputs)]
         if self._output_shapes is not None and len(self._output_shapes) == len(outs):
             outs = [o.view(s) if s and o.numel() == _numel(s) else o for o, s in zip(outs, self._output_shapes)]
         return outs
@@ -200,14 +234,20 @@ def build_wrapper(gm, ext) -> _DynamicCudaWrapper:
     input_param_names = _iter_placeholders_in_order(gm)
     selector_modules, reducer_mod = _collect_selector_modules(gm)
     selector_idx_tensors = [mod.idx for _, mod in selector_modules]
+    edge_permutation = None
     if reducer_mod is not None:
-        row_end_offsets, _ = _coo_rows_to_csr_ptr(reducer_mod.idx, int(reducer_mod.n))
+        row_ids = reducer_mod.idx.to(torch.int64)
+        if row_ids.numel() > 1 and bool((row_ids[1:] < row_ids[:-1]).any()):
+            row_ids, edge_permutation = torch.sort(row_ids, stable=True)
+            selector_idx_tensors = [t.index_select(0, edge_permutation.to(t.device)) for t in selector_idx_tensors]
+        row_end_offsets, _ = _coo_rows_to_csr_ptr(row_ids, int(reducer_mod.n))
     else:
         row_end_offsets = None
     gather_value_inputs = _infer_gather_value_inputs(gm, [q for q, _ in selector_modules])
     non_gather_value_inputs = [n for n in input_param_names if n not in gather_value_inputs]
     wrapper = _DynamicCudaWrapper(ext, input_param_names, non_gather_value_inputs, gather_value_inputs,
-                                  selector_idx_tensors, row_end_offsets, _output_shapes(gm), _written_inputs(gm))
+                                  selector_idx_tensors, row_end_offsets, _output_shapes(gm), _written_inputs(gm),
+                                  edge_permutation, _per_edge_outputs(gm))
     names = getattr(ext, "param_names", None)
     if callable(names):             # a library of this package knows its own argument list: cross-check
         expected = non_gather_value_inputs + gather_value_inputs

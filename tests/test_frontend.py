@@ -296,3 +296,44 @@ def test_reference_named_entry_point_writes_the_hip_source(tmp_path):
     assert path.endswith(".hip") and "flexspmv_launch" in text and "struct Graph" in text
     assert [p["name"] for p in signature["params"]][-3:] == ["row_end_offsets", "num_rows", "num_cols"]
     assert signature["index_inputs"] == ["selector_1_idx", "selector_2_idx"]
+
+
+def test_unsorted_reducer_rows_are_sorted_behind_the_wrapper():
+    """The reference's toy model draws its row ids unsorted (easier_spmv.py:126-127).  The wrapper sorts the
+    edges once, feeds the kernel sorted copies and puts per-edge results back in the model's edge order."""
+    class Unsorted(esr.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(3)
+            ne, nv, nr = 300, 40, 25
+            self.w = esr.Tensor(torch.rand(ne, 2, generator=g, dtype=torch.float64))
+            self.v = esr.Tensor(torch.rand(nv, 2, generator=g, dtype=torch.float64))
+            self.per_edge = esr.Tensor(torch.zeros(ne, 2, dtype=torch.float64))
+            self.per_row = esr.Tensor(torch.zeros(nr, 2, dtype=torch.float64))
+            self.total = esr.Tensor(torch.zeros(1, 2, dtype=torch.float64))
+            self.pick = esr.Selector(torch.randint(0, nv, (ne,), generator=g))
+            rows = torch.randint(0, nr, (ne,), generator=g)                               # not sorted
+            self.scatter = esr.Reducer(rows, nr)
+            self.row_of_edge = esr.Selector(rows)
+            self.per_edge_2 = esr.Tensor(torch.zeros(ne, 2, dtype=torch.float64))
+
+        def forward(self):
+            prod = self.pick(self.v) * self.w
+            self.per_edge[:] = prod
+            self.per_row[:] = self.scatter(prod)
+            self.total[:] = esr.sum(prod + self.w)
+            # a later kernel takes the per-edge value of the first one and gathers the fresh row sums
+            self.per_edge_2[:] = prod * self.row_of_edge(self.per_row)
+
+    eager, traced = Unsorted(), Unsorted()
+    assert bool((traced.scatter.idx[1:] < traced.scatter.idx[:-1]).any())
+    [compiled] = esr.compile([traced], "torch")
+    exts, skipped = replace_all_with_oracle(compiled, "t_unsorted")
+    assert not skipped
+    eager()
+    compiled()
+    assert torch.equal(eager.per_edge, traced.per_edge)                        # back in the model's edge order
+    assert torch.allclose(eager.per_edge_2, traced.per_edge_2, rtol=1e-13, atol=0)
+    assert len(exts) >= 3
+    assert torch.allclose(eager.per_row, traced.per_row, rtol=1e-13, atol=0)
+    assert torch.allclose(eager.total, traced.total, rtol=1e-13, atol=0)
