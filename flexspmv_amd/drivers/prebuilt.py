@@ -12,9 +12,9 @@ from .. import frontend as esr
 from ..ir import FusedGraphIR
 
 
-def _system(device="cpu", dtype=torch.float64):
+def _system(device="cpu", dtype=torch.float64, num_nnz=64, sorted_rows=True):
     from .system_model import make_system
-    return make_system(64, 17, 13, device=device, dtype=dtype)
+    return make_system(num_nnz, 17, 13, device=device, dtype=dtype, sorted_rows=sorted_rows)
 
 
 def _swe(device="cpu", dtype=torch.float64, points=900, dt=0.0005):

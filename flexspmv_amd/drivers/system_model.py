@@ -1,7 +1,7 @@
 """The toy ``System`` model of the reference's code-generation driver (easier_spmv.py:17-69): two
 selectors on one vertex tensor, edge tensors of item shape (2,1) and (2,3), two per-edge stores and one
-reducer.  The row ids are sorted here (the reference draws them unsorted, which its own COO -> CSR
-conversion cannot represent)."""
+reducer.  The row ids are sorted by default (the reference draws them unsorted, which its own COO -> CSR
+conversion cannot represent; ``sorted_rows=False`` reproduces that)."""
 from __future__ import annotations
 
 import torch
@@ -33,10 +33,14 @@ class System(esr.Module):
         self.y_reducer_1[:] = self.reducer_1(add_1)
 
 
-def make_system(num_nnz=20, num_cols=11, num_rows=11, device="cpu", dtype=torch.float64, seed=52) -> System:
+def make_system(num_nnz=20, num_cols=11, num_rows=11, device="cpu", dtype=torch.float64, seed=52,
+                sorted_rows=True) -> System:
     g = torch.Generator().manual_seed(seed)
     rnd = lambda *s: torch.rand(*s, generator=g, dtype=dtype).to(device)   # noqa: E731
-    rows = torch.sort(torch.randint(0, num_rows, (num_nnz,), generator=g)).values.to(device)
+    rows = torch.randint(0, num_rows, (num_nnz,), generator=g)
+    if sorted_rows:        # False: the reference's own set-up; the replacement wrapper then sorts the edges
+        rows = torch.sort(rows).values
+    rows = rows.to(device)
     col_1 = torch.randint(0, num_cols, (num_nnz,), generator=g).to(device)
     col_2 = torch.randint(0, num_cols, (num_nnz,), generator=g).to(device)
     return System(rnd(num_nnz, 2, 1), rnd(num_nnz, 2, 3), rnd(num_cols, 2, 1), col_1, col_2, rows,

@@ -42,6 +42,12 @@ def test_system_model_float64():
     assert torch.allclose(c.y_add_2.reshape(-1, 6), expected, rtol=1e-14, atol=0)
 
 
+def test_system_model_with_unsorted_rows():
+    """The reference's own set-up of the toy model: row ids in random order, sorted behind the wrapper."""
+    c = run("system", 2, 1e-12, skip=("y_add_2",), num_nnz=5000, sorted_rows=False)
+    assert bool((c.reducer_1.idx[1:] < c.reducer_1.idx[:-1]).any())
+
+
 def test_system_model_float32():
     run("system", 3, 1e-5, skip=("y_add_2",), dtype=torch.float32)
 
