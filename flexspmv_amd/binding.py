@@ -58,7 +58,7 @@ class LaunchArgs(ctypes.Structure):
 
 
 def load_library(path: str) -> ctypes.CDLL:
-    """dlopen a generated library and type its five entry points."""
+    """dlopen a generated library and type its entry points."""
     if not os.path.exists(path):
         raise RuntimeError(f"FlexSpmv library {path} is not built (run __graft_entry__.build())")
     try:

@@ -1,7 +1,7 @@
 /* C interface of a generated FlexSpmv library for MI355X (gfx950).
  *
  * One shared library is generated per fused sub-graph (select -> map -> reduce / aggregate).  Every
- * such library exports the same five symbols below; nothing in the signatures is a torch type, so
+ * such library exports the same six symbols below; nothing in the signatures is a torch type, so
  * any host (Python ctypes, a torch extension, C++) can bind them.
  *
  * What each entry point stands in for in the reference:
