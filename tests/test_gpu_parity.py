@@ -12,7 +12,7 @@ from flexspmv_amd import graphs
 from flexspmv_amd import workloads as W
 from flexspmv_amd.binding import load_named
 from oracle.runner import run_oracle
-from tests.util_inputs import STRUCTURES, make_inputs, row_structure
+from tests.util_inputs import STRUCTURES, make_inputs, random_row_structure, row_structure
 from tests.test_oracle_pins import op_zoo_inputs
 
 pytestmark = pytest.mark.gpu
@@ -119,6 +119,24 @@ def test_index_shuffle_map_only_int64(dtype):
     assert outs == []
     _, after = gpu_launch("bpoints_copy", tensors, None, nr, nc)
     assert np.array_equal(after["bp_1"], tensors["bpoints"][:, 1])
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_row_structures(seed):
+    """Forty random (sub-graph, dtype, row structure) combinations per seed against the oracle."""
+    rng = np.random.default_rng(seed)
+    names = REDUCER_GRAPHS + ["op_zoo"]
+    for case in range(40):
+        name = names[int(rng.integers(0, len(names)))]
+        dtype = [np.float32, np.float64][int(rng.integers(0, 2))]
+        row_ptr = random_row_structure(rng)
+        nr, ne = len(row_ptr) - 1, int(row_ptr[-1])
+        print(f"case random seed={seed} #{case} {name} {np.dtype(dtype).name} rows={nr} ne={ne}", flush=True)
+        if name == "op_zoo":
+            check_against_oracle(name, op_zoo_inputs(rng, ne, max(nr, 64), dtype), row_ptr, nr, max(nr, 64), dtype)
+        else:
+            tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get(name), dtype, rng, row_ptr=row_ptr)
+            check_against_oracle(name, tensors, row_ptr, nr, nc, dtype)
 
 
 def test_results_are_bitwise_reproducible():

@@ -43,6 +43,39 @@ def row_structure(kind, rng, tile=2048):
     return np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
 
 
+def random_row_structure(rng, max_edges=1_500_000):
+    """A row pointer drawn from eight families of row-length distributions (uniform short, uniform long,
+    heavy-tailed, constant, isolated giants, sparse rows between empty ones, around the row-path limit,
+    blocks of different character)."""
+    kind = int(rng.integers(0, 8))
+    n = int(rng.integers(1, 6000))
+    if kind == 0:
+        lens = rng.integers(0, 4, n)
+    elif kind == 1:
+        lens = rng.integers(0, 40, n)
+    elif kind == 2:
+        lens = (rng.pareto(1.1, n) * rng.integers(1, 20)).astype(np.int64)
+    elif kind == 3:
+        lens = np.full(n, int(rng.integers(1, 70)))
+    elif kind == 4:
+        lens = np.zeros(n, dtype=np.int64)
+        k = rng.integers(0, n, max(1, n // 50))
+        lens[k] = rng.integers(1, 5000, len(k))
+    elif kind == 5:
+        lens = rng.integers(0, 2, n) * rng.integers(1, 300, n)
+    elif kind == 6:
+        lens = rng.integers(28, 37, n)
+    else:
+        lens = np.concatenate([rng.integers(3, 8, n), np.zeros(int(rng.integers(0, 5000)), dtype=np.int64),
+                               rng.integers(0, 3, n)])
+    lens = lens.astype(np.int64)
+    if lens.sum() > max_edges:
+        lens = lens // (lens.sum() // max_edges + 1)
+    if lens.sum() == 0:
+        lens[-1] = 1
+    return np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+
+
 STRUCTURES = ["mesh", "mesh_with_gaps", "skewed", "one_long_row", "mostly_empty", "tiny", "exact_tiles", "len33",
               "empty_tiles", "uniform_30", "uneven_short", "rows_5"]
 
