@@ -266,8 +266,26 @@ class CompiledModule(fx.GraphModule):
             return getattr(original, name)
 
 
+def _drop_unused_values(graph: fx.Graph) -> None:
+    """Remove call nodes whose value nobody uses, except in-place stores (``x[:] = v``, ``x.copy_(v)``,
+    ``x.add_(v)``), which are kept for their effect.  (fx's own dead-code pass does not know that the
+    in-place methods have effects.)"""
+    changed = True
+    while changed:
+        changed = False
+        for node in reversed(list(graph.nodes)):
+            if node.op not in ("call_module", "call_function", "call_method", "get_attr") or node.users:
+                continue
+            store = (node.op == "call_function" and node.target in (operator.setitem, operator.iadd)) or \
+                    (node.op == "call_method" and isinstance(node.target, str) and node.target.endswith("_"))
+            if not store:
+                graph.erase_node(node)
+                changed = True
+
+
 def compile_module(model: nn.Module) -> CompiledModule:
     traced_graph = _Tracer().trace(model)
+    _drop_unused_values(traced_graph)
     gm = fx.GraphModule(model, traced_graph)
     propagate_meta(gm)
     groups = group_nodes(gm)

@@ -197,6 +197,8 @@ class GraphBuilder:
         for n in self._nodes:
             name = n["name"]
             shape = self._shape[name]
+            if n["kind"] in ("reducer", "sum") and name not in out_set:
+                continue        # a reduction nobody reads: it has no output buffer, so it is not generated
             if n["kind"] == "placeholder":
                 if name in out_set:
                     continue

@@ -23,9 +23,9 @@ Per function, what is followed and what pins it:
   Pinned by math.fsum and by the map-only instance in tests/golden/merge_kat.json.
 
 A sub-graph holding reducers AND aggregators has no single counterpart in the reference (its
-templates hold one or the other, codegen/merged_gen_cpu.py:87-89): the oracle runs the reducer pass,
-then the flat pass with in-place stores switched off, which is what running the reference's two
-kernels over the same inputs yields.
+templates hold one or the other, codegen/merged_gen_cpu.py:87-89): the oracle runs the flat pass with
+in-place stores switched off and then the reducer pass, which is what running the reference's two kernels
+over the same - original - inputs yields.
 """
 from __future__ import annotations
 
@@ -208,9 +208,11 @@ void flat_pass(int num_threads, void* const* vin, const int* const* iin, void* c
 """
     calls = []
     if red:
-        calls.append("reducer_pass<ValueT>(num_threads, row_ptr, vin, iin, out, num_rows, ne, true);")
+        # the aggregator pass runs first, with its stores off, so that it sees the inputs as the caller
+        # handed them over (the reducer pass may overwrite them through setitem / copy_ / add_)
         if agg:
             calls.append("flat_pass<ValueT>(num_threads, vin, iin, out, num_rows, ne, false);")
+        calls.append("reducer_pass<ValueT>(num_threads, row_ptr, vin, iin, out, num_rows, ne, true);")
     else:
         calls.append("flat_pass<ValueT>(num_threads, vin, iin, out, num_rows, ne, true);")
     src += f"""
