@@ -192,16 +192,16 @@ def _emit_selector(s: Dict[str, Any]) -> Tuple[List[str], List[str], List[str], 
     if s["selector"] == 1:
         name, idx = s["name"], f"column_indices_{s['name']}"
         return ([f"OffsetT {idx};"],
-                [f"f.{idx} = flex::stream_load(p.{s['selector_name']}_ptr + e);"],
+                [f"q_f.{idx} = flex::stream_load(q_p.{s['selector_name']}_idx_ptr + q_e);"],
                 [f"{T} {name};"],
-                [f"g.{name} = {T}(p.{s['target']}_ptr + (size_t)f.{idx} * {dim});"],
-                [f"{T} {name} = g.{name};"])
+                [f"q_g.{name} = {T}(q_p.{s['target']}_ptr + (size_t)q_f.{idx} * {dim});"],
+                [f"{T} {name} = q_g.{name};"])
     name = s["selector_name"]
     return ([f"{T} {name};"],
-            [f"f.{name}.values[{i}] = flex::stream_load(p.{s['target']}_ptr + (size_t)e * {dim} + {i});"
+            [f"q_f.{name}.values[{i}] = flex::stream_load(q_p.{s['target']}_ptr + (size_t)q_e * {dim} + {i});"
              for i in range(dim)],
             [], [],
-            [f"{T} {name} = f.{name};"])
+            [f"{T} {name} = q_f.{name};"])
 
 
 def _store_loop(ptr: str, edge: str, dim: int, src: str, src_dim: int) -> List[str]:
@@ -244,14 +244,14 @@ def _emit_map(op: Dict[str, Any], vars: Dict[str, Var], edge: str) -> List[str]:
     dim = get_dim_length(op["shape"])
     if o == "copy_":
         dst, src = a[0], a[1]
-        return _store_loop(f"p.{dst}_ptr", edge, dim, src, vars[src].dim)
+        return _store_loop(f"q_p.{dst}_ptr", edge, dim, src, vars[src].dim)
     if o == "add_":
         dst = a[0]
-        return [f"{dst} = {dst} + {a[1]};"] + _store_loop(f"p.{dst}_ptr", edge, dim, dst, vars[dst].dim)
+        return [f"{dst} = {dst} + {a[1]};"] + _store_loop(f"q_p.{dst}_ptr", edge, dim, dst, vars[dst].dim)
     if o == "setitem":
         dst, src = _arg(op["args"][0]), _arg(op["args"][2])
         sd = vars[src].dim
-        lines = _store_loop(f"p.{dst}_ptr", edge, dim, src, sd)
+        lines = _store_loop(f"q_p.{dst}_ptr", edge, dim, src, sd)
         lines += [f"{dst}.values[{i}] = {src}.values[{i % sd}];" for i in range(dim)]
         return lines
     raise ValueError(f"Operation {o} not supported")
@@ -303,13 +303,13 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
     params, fill = [], []
     for i, n in enumerate(plan.value_inputs):
         params.append(f"ValueT* __restrict__ {n}_ptr;")
-        fill.append(f"p.{n}_ptr = static_cast<ValueT*>(a->value_inputs[{i}]);")
+        fill.append(f"q_p.{n}_ptr = static_cast<ValueT*>(a->value_inputs[{i}]);")
     for i, s in enumerate(plan.selector_inputs):
-        params.append(f"const OffsetT* __restrict__ {s}_ptr;")
-        fill.append(f"p.{s}_ptr = a->index_inputs[{i}];")
+        params.append(f"const OffsetT* __restrict__ {s}_idx_ptr;")
+        fill.append(f"q_p.{s}_idx_ptr = a->index_inputs[{i}];")
     for i, o in enumerate(plan.outputs):
         params.append(f"ValueT* __restrict__ output_y_{o.name}_ptr;")
-        fill.append(f"p.output_y_{o.name}_ptr = static_cast<ValueT*>(a->outputs[{i}]);")
+        fill.append(f"q_p.output_y_{o.name}_ptr = static_cast<ValueT*>(a->outputs[{i}]);")
 
     # ---- typedefs -------------------------------------------------------------------------
     typedefs, seen = [], set()
@@ -344,10 +344,10 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         if var not in rebuilt:
             s2.append(f"{v.ctype} {var};" if v.kind == "tensor" else f"ValueT {var};")
             rebuilt.add(var)
-        s2.append(f"{_component(v, c)} = xch.v[{slot}];")
+        s2.append(f"{_component(v, c)} = q_xch.v[{slot}];")
     for sel, src, dim, first in kp.row_sources:
         s2.append(f"TensorInput_{src}_T {sel};")
-        s2 += [f"{sel}.values[{i}] = rv.v[{first + i}];" for i in range(dim)]
+        s2 += [f"{sel}.values[{i}] = q_rv.v[{first + i}];" for i in range(dim)]
 
     map_output_names = {o.name: o for o in plan.outputs if o.kind == "map"}
     for op_index, op in enumerate(map_ops):
@@ -356,20 +356,20 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
             continue
         stage = kp.op_stage.get(op_index, 1) if has_reducer else 1
         body = s1 if stage == 1 else s2
-        body.extend(_emit_map(op, kp.vars, "e"))
+        body.extend(_emit_map(op, kp.vars, "q_e"))
         if op["name"] in map_output_names:
             out = map_output_names[op["name"]]
             v = kp.vars[op["name"]]
             if v.kind == "scalar":
-                body.append(f"flex::stream_store(p.output_y_{out.name}_ptr + (size_t)e, {v.name});")
+                body.append(f"flex::stream_store(q_p.output_y_{out.name}_ptr + (size_t)q_e, {v.name});")
             else:
-                body.extend(_store_loop(f"p.output_y_{out.name}_ptr", "e", out.dim, v.name, v.dim))
+                body.extend(_store_loop(f"q_p.output_y_{out.name}_ptr", "q_e", out.dim, v.name, v.dim))
     # a map output may also be a (stage-1) selector / input variable
     for name, out in map_output_names.items():
         if not any(op["name"] == name for op in map_ops):
             v = kp.vars[name]
             (s1 if v.stage == 1 or not has_reducer else s2).extend(
-                _store_loop(f"p.output_y_{out.name}_ptr", "e", out.dim, v.name, v.dim))
+                _store_loop(f"q_p.output_y_{out.name}_ptr", "q_e", out.dim, v.name, v.dim))
 
     agg2_mask = 0
     stage1_has_agg = False
@@ -377,35 +377,35 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
     for (rname, first, dim), r in zip(kp.red_slices, red_ops):
         v = kp.vars[arg_name(r["args"][0])]
         for c in range(dim):
-            s2.append(f"tot.v[{first + c}] = {_component(v, c % v.dim)};")
+            s2.append(f"q_tot.v[{first + c}] = {_component(v, c % v.dim)};")
     # aggregator arguments
     for (gname, first, dim), g in zip(kp.agg_slices, agg_ops):
         v = kp.vars[arg_name(g["args"][0])]
         in_walk = has_reducer and v.final_stage == 2
         for c in range(dim):
             if in_walk:
-                s2.append(f"agg.v[{first + c}] = {_component(v, c % v.dim)};")
+                s2.append(f"q_agg.v[{first + c}] = {_component(v, c % v.dim)};")
                 agg2_mask |= 1 << (first + c)
             else:
-                s1.append(f"agg.v[{first + c}] += {_component(v, c % v.dim)};")
+                s1.append(f"q_agg.v[{first + c}] += {_component(v, c % v.dim)};")
                 stage1_has_agg = True
     # exchange writes close stage 1
     if has_reducer:
         for var, c, slot in kp.exchange:
-            s1.append(f"xch.v[{slot}] = {_component(kp.vars[var], c)};")
+            s1.append(f"q_xch.v[{slot}] = {_component(kp.vars[var], c)};")
 
     stage2_pure = not any("stream_store(" in line for line in s2)
     stage1_pure = not stage1_has_agg and not any("stream_store(" in line for line in s1)
     load_row, store_row, add_row, store_agg = [], [], [], []
     for sel, src, dim, first in kp.row_sources:
-        load_row += [f"rv.v[{first + i}] = p.{src}_ptr[(size_t)row * {dim} + {i}];" for i in range(dim)]
+        load_row += [f"q_rv.v[{first + i}] = q_p.{src}_ptr[(size_t)q_row * {dim} + {i}];" for i in range(dim)]
     for (rname, first, dim) in kp.red_slices:
         for c in range(dim):
-            store_row.append(f"flex::stream_store(p.output_y_{rname}_ptr + (size_t)row * {dim} + {c}, tot.v[{first + c}]);")
-            add_row.append(f"p.output_y_{rname}_ptr[(size_t)row * {dim} + {c}] += tot.v[{first + c}];")
+            store_row.append(f"flex::stream_store(q_p.output_y_{rname}_ptr + (size_t)q_row * {dim} + {c}, q_tot.v[{first + c}]);")
+            add_row.append(f"q_p.output_y_{rname}_ptr[(size_t)q_row * {dim} + {c}] += q_tot.v[{first + c}];")
     for (gname, first, dim) in kp.agg_slices:
         for c in range(dim):
-            store_agg.append(f"p.output_y_{gname}_ptr[{c}] = total.v[{first + c}];")
+            store_agg.append(f"q_p.output_y_{gname}_ptr[{c}] = q_total.v[{first + c}];")
 
     signature = generate_binding_code(None, inputs, outputs, selector_register)
     signature.update({
@@ -455,7 +455,7 @@ struct Graph {{
 {_indent(params)}  }};
 
 {_indent(typedefs, 2)}
-  static void fill(Params& p, const flexspmv_launch_args* a) {{
+  static void fill(Params& q_p, const flexspmv_launch_args* a) {{
 {_indent(fill)}  }}
 
   // streamed per-edge data (edge tensors and selector indices): first memory level
@@ -464,33 +464,33 @@ struct Graph {{
   // gathered vertex data: second memory level, addressed through Fetch
   struct Gather {{
 {_indent(gather_members)}  }};
-  static FLEX_DEV void fetch(const Params& p, const int e, Fetch& f) {{
+  static FLEX_DEV void fetch(const Params& q_p, const int q_e, Fetch& q_f) {{
 {_indent(fetch_body)}  }}
-  static FLEX_DEV void gather(const Params& p, const Fetch& f, Gather& g) {{
+  static FLEX_DEV void gather(const Params& q_p, const Fetch& q_f, Gather& q_g) {{
 {_indent(gather_body)}  }}
 
   // coalesced edge stage: the map on fetched + gathered data
   template <class X, class A>
-  static FLEX_DEV void stage1(const Params& p, const int e, const Fetch& f, const Gather& g, X& xch, A& agg) {{
+  static FLEX_DEV void stage1(const Params& q_p, const int q_e, const Fetch& q_f, const Gather& q_g, X& q_xch, A& q_agg) {{
 {_indent(s1)}  }}
 
   // merge-walk stage (row known): what edge e contributes to the reducers (tot) and to the
   // aggregators fed from the walk (agg); both are assigned, the kernel accumulates
   template <class X, class R, class T, class A>
-  static FLEX_DEV void contrib(const Params& p, const int e, const int row, const X& xch, const R& rv, T& tot, A& agg) {{
+  static FLEX_DEV void contrib(const Params& q_p, const int q_e, const int q_row, const X& q_xch, const R& q_rv, T& q_tot, A& q_agg) {{
 {_indent(s2)}  }}
 
   template <class R>
-  static FLEX_DEV void load_row(const Params& p, const int row, R& rv) {{
+  static FLEX_DEV void load_row(const Params& q_p, const int q_row, R& q_rv) {{
 {_indent(load_row)}  }}
   template <class T>
-  static FLEX_DEV void store_row(const Params& p, const int row, const T& tot) {{
+  static FLEX_DEV void store_row(const Params& q_p, const int q_row, const T& q_tot) {{
 {_indent(store_row)}  }}
   template <class T>
-  static FLEX_DEV void add_row(const Params& p, const int row, const T& tot) {{
+  static FLEX_DEV void add_row(const Params& q_p, const int q_row, const T& q_tot) {{
 {_indent(add_row)}  }}
   template <class A>
-  static FLEX_DEV void store_agg(const Params& p, const A& total) {{
+  static FLEX_DEV void store_agg(const Params& q_p, const A& q_total) {{
 {_indent(store_agg)}  }}
 }};
 

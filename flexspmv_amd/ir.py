@@ -44,6 +44,17 @@ _DTYPE_NAMES = {"float32": "float32", "float": "float32", "torch.float32": "floa
                 "int64": "int64", "long": "int64", "torch.int64": "int64"}
 
 
+# Node names become C++ locals of the generated code (as they do in the reference).  The generators keep
+# their own identifiers under the prefix ``q_``; what is left to refuse are C++ keywords and that prefix.
+RESERVED_NAMES = frozenset("""
+    alignas alignof and asm auto bool break case catch char class const constexpr continue decltype default
+    delete do double else enum explicit extern false float for friend goto if inline int long mutable
+    namespace new not nullptr operator or private protected public register return short signed sizeof static
+    struct switch template this throw true try typedef typename union unsigned using virtual void volatile
+    while xor flex oracle ValueT OffsetT
+""".split())
+
+
 def dtype_name(dtype: Any) -> str:
     """Canonical 'float32' | 'float64' | 'int64' for a torch/numpy dtype or its name."""
     key = str(dtype)
@@ -133,8 +144,15 @@ class GraphBuilder:
         shape = tuple(int(s) for s in shape)
         return shape if shape else (1,)
 
+    @staticmethod
+    def _check_name(name: str) -> None:
+        if name in RESERVED_NAMES or not name.isidentifier() or name.startswith(("__", "q_")):
+            raise ValueError(f"Operation on a value called {name!r} not supported: the name is not usable as a "
+                             "variable of the generated code")
+
     def placeholder(self, name: str, shape=(1,)) -> str:
         """A tensor argument of the fused sub-graph (edge tensor unless a selector gathers it)."""
+        self._check_name(name)
         self._shape[name] = self._shape_of(shape)
         self._nodes.append({"kind": "placeholder", "name": name})
         return name
@@ -142,6 +160,7 @@ class GraphBuilder:
     def select(self, name: str, source: str, module: Optional[str] = None,
                row_aligned: bool = False) -> str:
         """``name = <Selector module>(source)``: gather rows of ``source`` by the module's idx."""
+        self._check_name(name)
         self._shape[name] = self._shape[source]
         self._nodes.append({"kind": "selector", "name": name, "source": source,
                             "module": (module or name).replace(".", "_"),
@@ -154,12 +173,14 @@ class GraphBuilder:
             raise ValueError(f"Operation {op} not supported")
         if shape is None:
             shape = self._infer_shape(op, args)
+        self._check_name(name)
         self._shape[name] = self._shape_of(shape)
         self._nodes.append({"kind": "map", "op": op, "name": name, "args": list(args)})
         return name
 
     def reduce(self, name: str, arg: str, module: Optional[str] = None) -> str:
         """``name = <Reducer module>(arg)``: segment-sum by CSR row."""
+        self._check_name(name)
         self._shape[name] = self._shape[arg]
         self._nodes.append({"kind": "reducer", "name": name, "args": [arg],
                             "module": (module or name).replace(".", "_")})
@@ -167,6 +188,7 @@ class GraphBuilder:
 
     def aggregate(self, name: str, arg: str) -> str:
         """``name = sum(arg)`` over all edges."""
+        self._check_name(name)
         self._shape[name] = self._shape[arg]
         self._nodes.append({"kind": "sum", "name": name, "args": [arg]})
         return name
@@ -237,6 +259,8 @@ class GraphBuilder:
                 op, target = "call_function", "sum"
             elif n["kind"] == "map":
                 op, target = "call_function", n["op"]
+            elif n["kind"] == "selector":     # a gathered value handed on as it is: a per-edge (map) output
+                op, target = "call_module", n["module"]
             else:
                 raise ValueError(f"{name}: a {n['kind']} node cannot be a sub-graph output")
             outputs.append({"op": op, "name": name, "target": target, "dtype": "ValueT",

@@ -55,15 +55,15 @@ def _selector_statements(selector_register) -> List[str]:
     for s in selector_register:
         dim = get_dim_length(s["shape"])
         if s["selector"] == 1:   # gathered vertex tensor                       merged_gen_core.py:98-108
-            out.append(f"const int column_indices_{s['name']} = {s['selector_name']}_ptr[e];")
+            out.append(f"const int column_indices_{s['name']} = {s['selector_name']}_idx_ptr[q_e];")
             out.append(f"TensorInput_{s['target']}_T {s['name']}({s['target']}_ptr + (long)column_indices_{s['name']} * {dim});")
         else:                    # tensor streamed by edge id                   merged_gen_core.py:109-114
-            out.append(f"TensorInput_{s['target']}_T {s['selector_name']}({s['target']}_ptr + (long)e * {dim});")
+            out.append(f"TensorInput_{s['target']}_T {s['selector_name']}({s['target']}_ptr + (long)q_e * {dim});")
     return out
 
 
 def _store(ptr: str, dim: int, src: str) -> List[str]:
-    return [f"if (stores) for (int i = 0; i < {dim}; i++) {ptr}[(long)e * {dim} + i] = {src}.values[i];"]
+    return [f"if (q_stores) for (int q_i = 0; q_i < {dim}; q_i++) {ptr}[(long)q_e * {dim} + q_i] = {src}.values[q_i];"]
 
 
 def _map_statements(map_ops) -> List[str]:
@@ -96,7 +96,7 @@ def _map_statements(map_ops) -> List[str]:
         elif o == "setitem":                                                  # :202-213
             dst, src = _lit(op["args"][0]), _lit(op["args"][2])
             out += _store(f"{dst}_ptr", dim, src)
-            out.append(f"for (int i = 0; i < {dim}; i++) {dst}.values[i] = {src}.values[i];")
+            out.append(f"for (int q_i = 0; q_i < {dim}; q_i++) {dst}.values[q_i] = {src}.values[q_i];")
         elif o in ("reducer", "sum"):                                         # :184-185, :214-215
             continue
         else:
@@ -112,7 +112,7 @@ def generate_oracle_source(ir: FusedGraphIR) -> str:
     for i, n in enumerate(plan.value_inputs):
         unpack.append(f"ValueT* {n}_ptr = static_cast<ValueT*>(vin[{i}]);")
     for i, s in enumerate(plan.selector_inputs):
-        unpack.append(f"const int* {s}_ptr = iin[{i}];")
+        unpack.append(f"const int* {s}_idx_ptr = iin[{i}];")
     for i, o in enumerate(plan.outputs):
         unpack.append(f"ValueT* output_y_{o.name}_ptr = static_cast<ValueT*>(out[{i}]);")
     unpack = [u + " (void)" + u.split("=")[0].split()[-1] + ";" for u in unpack]
@@ -134,7 +134,7 @@ def generate_oracle_source(ir: FusedGraphIR) -> str:
     for o in plan.outputs:                                             # merged_gen_core.py:83-89
         if o.kind == "map":
             if o.name in norm_names:
-                body.append(f"if (stores) output_y_{o.name}_ptr[e] = {o.name};")
+                body.append(f"if (q_stores) output_y_{o.name}_ptr[q_e] = {o.name};")
             else:
                 body += _store(f"output_y_{o.name}_ptr", o.dim, o.name)
     body_txt = "\n".join("        " + b for b in body)
@@ -158,7 +158,7 @@ namespace {{
 // Reducer pass: cpu_template/merged_spmv_template_reducer.h:92-169.
 template <typename ValueT>
 void reducer_pass(int num_threads, const int* row_ptr, void* const* vin, const int* const* iin,
-                  void* const* out, int num_rows, int nnz, const bool stores) {{
+                  void* const* out, int num_rows, int nnz, const bool q_stores) {{
   const int* row_end = row_ptr + 1;                                             // :97
 {pad(unpack, 2)}
 {pad(typedefs, 2)}
@@ -166,17 +166,17 @@ void reducer_pass(int num_threads, const int* row_ptr, void* const* vin, const i
 #pragma omp parallel for schedule(static) num_threads(num_threads)
   for (int tid = 0; tid < num_threads; tid++) {{
     const Span span = reducer_thread_span(tid, num_threads, row_end, num_rows, nnz);   // :101-121
-    int e = span.begin.y;
-    for (int row = span.begin.x; row < span.end.x; ++row) {{                     // whole rows :124-144
+    int q_e = span.begin.y;
+    for (int q_row = span.begin.x; q_row < span.end.x; ++q_row) {{                     // whole rows :124-144
 {pad([f'TensorOutput_{n}_T reducer_{n}_running_total;' for n, _, _ in red], 6)}
-      for (; e < row_end[row]; ++e) {{
+      for (; q_e < row_end[q_row]; ++q_e) {{
 {body_txt}
 {pad([f'reducer_{n}_running_total += {a};' for n, _, a in red], 8)}
       }}
-{pad([f'for (int i = 0; i < {d}; i++) output_y_{n}_ptr[(long)row * {d} + i] = reducer_{n}_running_total.values[i];' for n, d, _ in red], 6)}
+{pad([f'for (int q_i = 0; q_i < {d}; q_i++) output_y_{n}_ptr[(long)q_row * {d} + q_i] = reducer_{n}_running_total.values[q_i];' for n, d, _ in red], 6)}
     }}
 {pad([f'TensorOutput_{n}_T {n}_running_total_partial;' for n, _, _ in red], 4)}
-    for (; e < span.end.y; ++e) {{                                               // open last row :147-160
+    for (; q_e < span.end.y; ++q_e) {{                                               // open last row :147-160
 {body_txt}
 {pad([f'{n}_running_total_partial += {a};' for n, _, a in red], 6)}
     }}
@@ -190,7 +190,7 @@ void reducer_pass(int num_threads, const int* row_ptr, void* const* vin, const i
 // Flat pass (aggregators and map-only): cpu_template/merged_spmv_template_aggregator.h:92-136.
 template <typename ValueT>
 void flat_pass(int num_threads, void* const* vin, const int* const* iin, void* const* out,
-               int num_rows, int nnz, const bool stores) {{
+               int num_rows, int nnz, const bool q_stores) {{
 {pad(unpack, 2)}
 {pad(typedefs, 2)}
 {pad([f'std::vector<TensorOutput_{n}_T> {n}_running_carry_out(num_threads);' for n, _, _ in agg], 2)}
@@ -198,7 +198,7 @@ void flat_pass(int num_threads, void* const* vin, const int* const* iin, void* c
   for (int tid = 0; tid < num_threads; tid++) {{
     int first, last;
     flat_thread_range(tid, num_threads, num_rows, nnz, first, last);            // :99-111
-    for (int e = first; e < last; ++e) {{
+    for (int q_e = first; q_e < last; ++q_e) {{
 {body_txt}
 {pad([f'{n}_running_carry_out[tid] += {a};' for n, _, a in agg], 6)}
     }}

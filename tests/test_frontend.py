@@ -458,3 +458,49 @@ def test_aggregator_sees_the_inputs_as_handed_over_when_the_same_kernel_overwrit
         compiled()
     for k in ("a", "rows", "total"):
         assert torch.allclose(getattr(eager, k), getattr(traced, k), rtol=1e-13, atol=0), k
+
+
+def test_tensor_names_that_look_like_kernel_internals_and_a_gathered_output():
+    """Model tensors called ``e``, ``total``, ``row`` or ``p`` and a selector whose node shares the name of a
+    value handed on to a later kernel must not collide with anything in the generated code (the generators
+    keep their own identifiers under ``q_`` and index pointers under ``<module>_idx_ptr``); a gathered value
+    may itself be a per-edge output."""
+    class Names(esr.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(8)
+            self.p = esr.Tensor(torch.rand(12, 2, generator=g, dtype=torch.float64))
+            self.e = esr.Tensor(torch.zeros(50, 2, dtype=torch.float64))
+            self.total = esr.Tensor(torch.zeros(12, 2, dtype=torch.float64))
+            self.row = esr.Tensor(torch.rand(50, 2, generator=g, dtype=torch.float64))
+            self.sel = esr.Selector(torch.randint(0, 12, (50,), generator=g))
+            self.red = esr.Reducer(torch.sort(torch.randint(0, 12, (50,), generator=g)).values, 12)
+
+        def forward(self):
+            s = self.sel(self.p)
+            self.e[:] = s * self.row
+            self.total[:] = self.red(s)
+            self.p[:] = self.total * 0.5
+            self.e.add_(s * self.sel(self.p))          # s crosses into a later kernel as a placeholder "sel"
+
+    eager, traced = Names(), Names()
+    [compiled] = esr.compile([traced], "torch")
+    irs, skipped = lower_submodules(compiled, "t_names")
+    assert not skipped
+    first = irs[fused_call_nodes(compiled)[0].name]
+    assert any(o["name"] == "sel" and o["op"] == "call_module" for o in first.outputs)
+    from flexspmv_amd.codegen.merged_gen_gpu import generate_hip_source
+    for ir in irs.values():
+        text, _ = generate_hip_source(ir)
+        assert "q_p." in text and ("_idx_ptr" in text or not ir.inputs or all(i["dtype"] != "int" for i in ir.inputs))
+    exts, _ = replace_all_with_oracle(compiled, "t_names")
+    for _ in range(2):
+        eager()
+        compiled()
+    for (k, a), (_, b) in zip(eager.named_parameters(), traced.named_parameters()):
+        assert torch.allclose(a, b, rtol=1e-13, atol=0), k
+    with pytest.raises(ValueError, match="not usable"):
+        from flexspmv_amd.ir import GraphBuilder
+        GraphBuilder("bad").placeholder("q_e")
+    with pytest.raises(ValueError, match="not usable"):
+        GraphBuilder("bad").placeholder("double")
