@@ -110,11 +110,11 @@ def generate_oracle_source(ir: FusedGraphIR) -> str:
 
     unpack = []
     for i, n in enumerate(plan.value_inputs):
-        unpack.append(f"ValueT* {n}_ptr = static_cast<ValueT*>(vin[{i}]);")
+        unpack.append(f"ValueT* {n}_ptr = static_cast<ValueT*>(q_vin[{i}]);")
     for i, s in enumerate(plan.selector_inputs):
-        unpack.append(f"const int* {s}_idx_ptr = iin[{i}];")
+        unpack.append(f"const int* {s}_idx_ptr = q_iin[{i}];")
     for i, o in enumerate(plan.outputs):
-        unpack.append(f"ValueT* output_y_{o.name}_ptr = static_cast<ValueT*>(out[{i}]);")
+        unpack.append(f"ValueT* output_y_{o.name}_ptr = static_cast<ValueT*>(q_out[{i}]);")
     unpack = [u + " (void)" + u.split("=")[0].split()[-1] + ";" for u in unpack]
 
     typedefs, seen = [], set()
@@ -157,53 +157,53 @@ namespace {{
         src += f"""
 // Reducer pass: cpu_template/merged_spmv_template_reducer.h:92-169.
 template <typename ValueT>
-void reducer_pass(int num_threads, const int* row_ptr, void* const* vin, const int* const* iin,
-                  void* const* out, int num_rows, int nnz, const bool q_stores) {{
-  const int* row_end = row_ptr + 1;                                             // :97
+void reducer_pass(int q_num_threads, const int* q_row_ptr, void* const* q_vin, const int* const* q_iin,
+                  void* const* q_out, int q_num_rows, int q_nnz, const bool q_stores) {{
+  const int* q_row_end = q_row_ptr + 1;                                             // :97
 {pad(unpack, 2)}
 {pad(typedefs, 2)}
-{pad([f'std::vector<int> row_carry_out_{n}(num_threads); std::vector<TensorOutput_{n}_T> value_carry_out_{n}(num_threads);' for n, _, _ in red], 2)}
-#pragma omp parallel for schedule(static) num_threads(num_threads)
-  for (int tid = 0; tid < num_threads; tid++) {{
-    const Span span = reducer_thread_span(tid, num_threads, row_end, num_rows, nnz);   // :101-121
-    int q_e = span.begin.y;
-    for (int q_row = span.begin.x; q_row < span.end.x; ++q_row) {{                     // whole rows :124-144
+{pad([f'std::vector<int> row_carry_out_{n}(q_num_threads); std::vector<TensorOutput_{n}_T> value_carry_out_{n}(q_num_threads);' for n, _, _ in red], 2)}
+#pragma omp parallel for schedule(static) num_threads(q_num_threads)
+  for (int q_tid = 0; q_tid < q_num_threads; q_tid++) {{
+    const Span q_span = reducer_thread_span(q_tid, q_num_threads, q_row_end, q_num_rows, q_nnz);   // :101-121
+    int q_e = q_span.begin.y;
+    for (int q_row = q_span.begin.x; q_row < q_span.end.x; ++q_row) {{                     // whole rows :124-144
 {pad([f'TensorOutput_{n}_T reducer_{n}_running_total;' for n, _, _ in red], 6)}
-      for (; q_e < row_end[q_row]; ++q_e) {{
+      for (; q_e < q_row_end[q_row]; ++q_e) {{
 {body_txt}
 {pad([f'reducer_{n}_running_total += {a};' for n, _, a in red], 8)}
       }}
 {pad([f'for (int q_i = 0; q_i < {d}; q_i++) output_y_{n}_ptr[(long)q_row * {d} + q_i] = reducer_{n}_running_total.values[q_i];' for n, d, _ in red], 6)}
     }}
 {pad([f'TensorOutput_{n}_T {n}_running_total_partial;' for n, _, _ in red], 4)}
-    for (; q_e < span.end.y; ++q_e) {{                                               // open last row :147-160
+    for (; q_e < q_span.end.y; ++q_e) {{                                               // open last row :147-160
 {body_txt}
 {pad([f'{n}_running_total_partial += {a};' for n, _, a in red], 6)}
     }}
-{pad([f'row_carry_out_{n}[tid] = span.end.x; value_carry_out_{n}[tid] = {n}_running_total_partial;' for n, _, _ in red], 4)}
+{pad([f'row_carry_out_{n}[q_tid] = q_span.end.x; value_carry_out_{n}[q_tid] = {n}_running_total_partial;' for n, _, _ in red], 4)}
   }}
-{pad([f'reducer_carry_fixup<ValueT, {d}>(num_threads, num_rows, row_carry_out_{n}.data(), value_carry_out_{n}.data(), output_y_{n}_ptr);' for n, d, _ in red], 2)}
+{pad([f'reducer_carry_fixup<ValueT, {d}>(q_num_threads, q_num_rows, row_carry_out_{n}.data(), value_carry_out_{n}.data(), output_y_{n}_ptr);' for n, d, _ in red], 2)}
 }}
 """
     if agg or not red:
         src += f"""
 // Flat pass (aggregators and map-only): cpu_template/merged_spmv_template_aggregator.h:92-136.
 template <typename ValueT>
-void flat_pass(int num_threads, void* const* vin, const int* const* iin, void* const* out,
-               int num_rows, int nnz, const bool q_stores) {{
+void flat_pass(int q_num_threads, void* const* q_vin, const int* const* q_iin, void* const* q_out,
+               int q_num_rows, int q_nnz, const bool q_stores) {{
 {pad(unpack, 2)}
 {pad(typedefs, 2)}
-{pad([f'std::vector<TensorOutput_{n}_T> {n}_running_carry_out(num_threads);' for n, _, _ in agg], 2)}
-#pragma omp parallel for schedule(static) num_threads(num_threads)
-  for (int tid = 0; tid < num_threads; tid++) {{
-    int first, last;
-    flat_thread_range(tid, num_threads, num_rows, nnz, first, last);            // :99-111
-    for (int q_e = first; q_e < last; ++q_e) {{
+{pad([f'std::vector<TensorOutput_{n}_T> {n}_running_carry_out(q_num_threads);' for n, _, _ in agg], 2)}
+#pragma omp parallel for schedule(static) num_threads(q_num_threads)
+  for (int q_tid = 0; q_tid < q_num_threads; q_tid++) {{
+    int q_first, q_last;
+    flat_thread_range(q_tid, q_num_threads, q_num_rows, q_nnz, q_first, q_last);            // :99-111
+    for (int q_e = q_first; q_e < q_last; ++q_e) {{
 {body_txt}
-{pad([f'{n}_running_carry_out[tid] += {a};' for n, _, a in agg], 6)}
+{pad([f'{n}_running_carry_out[q_tid] += {a};' for n, _, a in agg], 6)}
     }}
   }}
-{pad([f'aggregator_fixup<ValueT, {d}>(num_threads, {n}_running_carry_out.data(), output_y_{n}_ptr);' for n, d, _ in agg], 2)}
+{pad([f'aggregator_fixup<ValueT, {d}>(q_num_threads, {n}_running_carry_out.data(), output_y_{n}_ptr);' for n, d, _ in agg], 2)}
 }}
 """
     calls = []
@@ -211,14 +211,14 @@ void flat_pass(int num_threads, void* const* vin, const int* const* iin, void* c
         # the aggregator pass runs first, with its stores off, so that it sees the inputs as the caller
         # handed them over (the reducer pass may overwrite them through setitem / copy_ / add_)
         if agg:
-            calls.append("flat_pass<ValueT>(num_threads, vin, iin, out, num_rows, ne, false);")
-        calls.append("reducer_pass<ValueT>(num_threads, row_ptr, vin, iin, out, num_rows, ne, true);")
+            calls.append("flat_pass<ValueT>(q_num_threads, q_vin, q_iin, q_out, q_num_rows, q_ne, false);")
+        calls.append("reducer_pass<ValueT>(q_num_threads, q_row_ptr, q_vin, q_iin, q_out, q_num_rows, q_ne, true);")
     else:
-        calls.append("flat_pass<ValueT>(num_threads, vin, iin, out, num_rows, ne, true);")
+        calls.append("flat_pass<ValueT>(q_num_threads, q_vin, q_iin, q_out, q_num_rows, q_ne, true);")
     src += f"""
 template <typename ValueT>
-void run_all(int num_threads, const int* row_ptr, void* const* vin, const int* const* iin,
-             void* const* out, int num_rows, int ne) {{
+void run_all(int q_num_threads, const int* q_row_ptr, void* const* q_vin, const int* const* q_iin,
+             void* const* q_out, int q_num_rows, int q_ne) {{
 {pad(calls, 2)}
 }}
 
@@ -226,13 +226,13 @@ void run_all(int num_threads, const int* row_ptr, void* const* vin, const int* c
 
 // dtype: 0 float, 1 double, 2 long.  Pointer arrays are in binding order.  Returns 0, or -1 for a bad
 // dtype, -2 when num_threads exceeds the reference's 256-entry carry arrays.
-extern "C" int oracle_run(int dtype, int num_threads, void* const* vin, const int* const* iin,
-                          void* const* out, const int* row_ptr, int num_rows, int ne) {{
-  if (num_threads < 1 || num_threads > 256) return -2;
+extern "C" int oracle_run(int dtype, int q_num_threads, void* const* q_vin, const int* const* q_iin,
+                          void* const* q_out, const int* q_row_ptr, int q_num_rows, int q_ne) {{
+  if (q_num_threads < 1 || q_num_threads > 256) return -2;
   switch (dtype) {{
-    case 0: run_all<float>(num_threads, row_ptr, vin, iin, out, num_rows, ne); return 0;
-    case 1: run_all<double>(num_threads, row_ptr, vin, iin, out, num_rows, ne); return 0;
-{"    case 2: run_all<long>(num_threads, row_ptr, vin, iin, out, num_rows, ne); return 0;" if plan.allow_int64 else ""}
+    case 0: run_all<float>(q_num_threads, q_row_ptr, q_vin, q_iin, q_out, q_num_rows, q_ne); return 0;
+    case 1: run_all<double>(q_num_threads, q_row_ptr, q_vin, q_iin, q_out, q_num_rows, q_ne); return 0;
+{"    case 2: run_all<long>(q_num_threads, q_row_ptr, q_vin, q_iin, q_out, q_num_rows, q_ne); return 0;" if plan.allow_int64 else ""}
     default: return -1;
   }}
 }}
