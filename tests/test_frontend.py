@@ -339,53 +339,88 @@ def test_unsorted_reducer_rows_are_sorted_behind_the_wrapper():
     assert torch.allclose(eager.total, traced.total, rtol=1e-13, atol=0)
 
 
-def _random_model_source(rng, n_stmts=14):
+def _random_model_source(rng, n_stmts=14, rich=False):
     """Python source of a random model: gathers, per-edge and per-vertex arithmetic, reductions, in-place
-    stores and re-reads of model tensors, in random order."""
+    stores and re-reads of model tensors, in random order.  ``rich`` adds the rest of the operation set
+    (neg, abs, powers, exp, division, comparisons with where, norm, column picks with clone / copy_)."""
     lines = []
-    edge_vals, vert_vals = [], []
+    edge_vals, vert_vals, edge_cols, vert_cols = [], [], [], []
     counter = [0]
 
     def fresh(prefix):
         counter[0] += 1
         return f"{prefix}{counter[0]}"
 
-    def edge_operand():
-        pool = edge_vals + [f"self.E{i}" for i in range(3)]
+    def pick(pool):
         return pool[int(rng.integers(0, len(pool)))]
+
+    def edge_operand():
+        return pick(edge_vals + [f"self.E{i}" for i in range(3)])
 
     def vert_operand():
-        pool = vert_vals + [f"self.V{i}" for i in range(3)]
-        return pool[int(rng.integers(0, len(pool)))]
+        return pick(vert_vals + [f"self.V{i}" for i in range(3)])
+
+    def unary(x):
+        k = int(rng.integers(0, 7))
+        return [f"-{x}", f"abs({x} - 0.5)", f"{x} ** 2", f"({x} * {x} + 0.5) ** 0.5", f"torch.exp(-({x} * {x}))",
+                f"{x} / ({x} * {x} + 1.0)", f"esr.norm({x}) * {x}"][k]
+
+    def binary(a, b):
+        k = int(rng.integers(0, 4))
+        return [f"torch.where({a} > {b}, {a}, {b})", f"torch.where({a} < {b}, {a}, {b} * 0.5)", f"{a} / ({b} * {b} + 1.0)",
+                f"{a} * {b} - {a}"][k]
 
     for _ in range(n_stmts):
-        kind = int(rng.integers(0, 9))
+        kind = int(rng.integers(0, 14 if rich else 9))
         if kind <= 1:
             name = fresh("e")
             lines.append(f"{name} = self.sel{int(rng.integers(0, 2))}({vert_operand()})")
             edge_vals.append(name)
         elif kind == 2:
             name = fresh("e")
-            op = "+-*"[int(rng.integers(0, 3))]
-            lines.append(f"{name} = {edge_operand()} {op} {edge_operand()}")
+            lines.append(f"{name} = {edge_operand()} {'+-*'[int(rng.integers(0, 3))]} {edge_operand()}")
             edge_vals.append(name)
         elif kind == 3:
             name = fresh("v")
-            op = "+-*"[int(rng.integers(0, 3))]
-            lines.append(f"{name} = {vert_operand()} {op} {vert_operand()}")
+            lines.append(f"{name} = {vert_operand()} {'+-*'[int(rng.integers(0, 3))]} {vert_operand()}")
             vert_vals.append(name)
         elif kind == 4 and edge_vals:
             name = fresh("v")
-            lines.append(f"{name} = self.red({edge_vals[int(rng.integers(0, len(edge_vals)))]})")
+            lines.append(f"{name} = self.red({pick(edge_vals)})")
             vert_vals.append(name)
         elif kind == 5 and vert_vals:
-            lines.append(f"self.V{int(rng.integers(0, 3))}[:] = {vert_vals[int(rng.integers(0, len(vert_vals)))]} * 0.5")
+            lines.append(f"self.V{int(rng.integers(0, 3))}[:] = {pick(vert_vals)} * 0.5")
         elif kind == 6 and edge_vals:
-            lines.append(f"self.E{int(rng.integers(0, 3))}[:] = {edge_vals[int(rng.integers(0, len(edge_vals)))]} * 0.5")
+            lines.append(f"self.E{int(rng.integers(0, 3))}[:] = {pick(edge_vals)} * 0.5")
         elif kind == 7 and vert_vals:
-            lines.append(f"self.V{int(rng.integers(0, 3))}.add_({vert_vals[int(rng.integers(0, len(vert_vals)))]} * 0.25)")
+            lines.append(f"self.V{int(rng.integers(0, 3))}.add_({pick(vert_vals)} * 0.25)")
         elif kind == 8 and edge_vals:
-            lines.append(f"self.S[:] = esr.sum({edge_vals[int(rng.integers(0, len(edge_vals)))]})")
+            lines.append(f"self.S[:] = esr.sum({pick(edge_vals)})")
+        elif kind == 9:
+            name = fresh("e")
+            lines.append(f"{name} = {unary(edge_operand())}")
+            edge_vals.append(name)
+        elif kind == 10:
+            name = fresh("v")
+            lines.append(f"{name} = {binary(vert_operand(), vert_operand())}")
+            vert_vals.append(name)
+        elif kind == 11:
+            name = fresh("e")
+            lines.append(f"{name} = {binary(edge_operand(), edge_operand())}")
+            edge_vals.append(name)
+        elif kind == 12:                      # column picks: (n, 2) -> (n,), stored into 1-D tensors
+            name = fresh("c")
+            lines.append(f"{name} = {edge_operand()}[:, {int(rng.integers(0, 2))}].clone()")
+            edge_cols.append(name)
+            if len(edge_cols) > 1 and rng.random() < 0.5:
+                lines.append(f"self.EC.copy_({pick(edge_cols)} * {pick(edge_cols)})")
+            else:
+                lines.append(f"self.EC[:] = {name} * 0.5")
+        elif kind == 13:
+            name = fresh("d")
+            lines.append(f"{name} = {vert_operand()}[:, {int(rng.integers(0, 2))}].clone()")
+            vert_cols.append(name)
+            lines.append(f"self.VC.copy_({name})")
     if not any(l.startswith("self.") for l in lines):
         lines.append("self.V0[:] = self.V1 * 0.5")
     body = "\n".join("        " + l for l in lines)
@@ -398,6 +433,8 @@ class Random(esr.Module):
         for i in range(3):
             setattr(self, f"E{{i}}", esr.Tensor(torch.rand(ne, 2, generator=g, dtype=torch.float64)))
             setattr(self, f"V{{i}}", esr.Tensor(torch.rand(nv, 2, generator=g, dtype=torch.float64)))
+        self.EC = esr.Tensor(torch.zeros(ne, dtype=torch.float64))
+        self.VC = esr.Tensor(torch.zeros(nv, dtype=torch.float64))
         self.S = esr.Tensor(torch.zeros(1, 2, dtype=torch.float64))
         self.sel0 = esr.Selector(torch.randint(0, nv, (ne,), generator=g))
         self.sel1 = esr.Selector(torch.randint(0, nv, (ne,), generator=g))
@@ -414,7 +451,7 @@ def test_random_models_compile_to_the_same_results(seed):
     bit for bit over three steps (reads before and after in-place stores, gathers of freshly stored
     tensors, reductions feeding later gathers)."""
     rng = np.random.default_rng(1000 + seed)
-    source = _random_model_source(rng)
+    source = _random_model_source(rng, n_stmts=16, rich=(seed % 2 == 1))
     scope = {"esr": esr, "torch": torch}
     exec(source, scope)
     eager, traced = scope["Random"](), scope["Random"]()
