@@ -139,6 +139,21 @@ def test_random_row_structures(seed):
             check_against_oracle(name, tensors, row_ptr, nr, nc, dtype)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_reference_harness_default_problem(dtype):
+    """The default problem of the reference's CUDA harness (src/flex_spmv_full_red.cu:624-635): 1543 vertices,
+    123134 edges, 12314 rows, item widths 2 / 2 / 6, random sorted row offsets with empty rows - on the
+    sub-graph of its toy model - and of its CPU harness (main.cpp: 3241 rows, 324123 non-zeros, seed 12)."""
+    for rows, ne, seed in ((12314, 123134, 49), (3241, 324123, 12)):
+        rng = np.random.default_rng(seed)
+        cuts = np.sort(rng.integers(0, ne + 1, rows - 1))
+        row_ptr = np.concatenate([[0], cuts, [ne]]).astype(np.int32)
+        tensors, row_ptr, nr, nc, _ = make_inputs(graphs.get("system_two_selectors"), dtype, rng, row_ptr=row_ptr,
+                                                  positive=False)
+        print(f"case harness rows={rows} ne={ne} {np.dtype(dtype).name}", flush=True)
+        check_against_oracle("system_two_selectors", tensors, row_ptr, nr, nc, dtype)
+
+
 def test_results_are_bitwise_reproducible():
     rng = np.random.default_rng(9)
     row_ptr = row_structure("skewed", rng)
