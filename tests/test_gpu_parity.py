@@ -302,6 +302,53 @@ def test_shallow_water_1m_points_conservation_and_lake_at_rest():
     assert float(fu[~interior].abs().max()) > 0              # wall cells do feel the missing face
 
 
+def test_largest_supported_size_poisson_644_cubed():
+    """2.134e9 merge items (rows + non-zeros), 99.4 % of what 32-bit offsets allow: the 7-point operator on
+    a 644^3 grid, assembled on the device, against the stencil applied with dense shifts; one size
+    larger is refused with the reference's error."""
+    n, dev = 644, "cuda"
+    N = n ** 3
+    i = torch.arange(N, device=dev, dtype=torch.int64)
+    x_, y_, z_ = i % n, (i // n) % n, i // (n * n)
+    offs = [(-n * n, z_ > 0), (-n, y_ > 0), (-1, x_ > 0), (0, None), (1, x_ < n - 1), (n, y_ < n - 1), (n * n, z_ < n - 1)]
+    cnt = torch.zeros(N, device=dev, dtype=torch.int64)
+    for _, m in offs:
+        cnt += 1 if m is None else m.to(torch.int64)
+    ptr = torch.zeros(N + 1, device=dev, dtype=torch.int64)
+    torch.cumsum(cnt, 0, out=ptr[1:])
+    nnz = int(ptr[-1])
+    assert N + nnz == 2134231456
+    cols = torch.empty(nnz, device=dev, dtype=torch.int32)
+    vals = torch.empty(nnz, device=dev, dtype=torch.float64)
+    pos = ptr[:-1].clone()
+    for o, m in offs:
+        sel = i if m is None else m.nonzero().squeeze(1)
+        cols[pos[sel]] = (sel + o).to(torch.int32)
+        vals[pos[sel]] = 6.0 if o == 0 else -1.0
+        pos[sel] += 1
+    rows = torch.repeat_interleave(torch.arange(N, device=dev, dtype=torch.int32), cnt)
+    del pos, cnt, x_, y_, z_, offs, sel, i
+    x = torch.rand(N, device=dev, dtype=torch.float64) * 2 - 1
+    ext = load_named("spmv_dot", build_if_missing=False)
+    given = {"vals": vals, "x": x, "selector_col_idx": cols, "selector_row_idx": rows,
+             "row_end_offsets": ptr.to(torch.int32), "num_rows": N, "num_cols": N}
+    print(f"case largest size rows={N} nnz={nnz}", flush=True)
+    y, dot = ext.merged_spmv_launch(*[given[k] for k in ext.param_names()])
+    xb = x.view(n, n, n)
+    ref = 6 * xb.clone()
+    ref[1:] -= xb[:-1]; ref[:-1] -= xb[1:]
+    ref[:, 1:] -= xb[:, :-1]; ref[:, :-1] -= xb[:, 1:]
+    ref[:, :, 1:] -= xb[:, :, :-1]; ref[:, :, :-1] -= xb[:, :, 1:]
+    assert (y.view_as(ref) - ref).abs().max().item() <= 1e-12 * 12
+    d_ref = (xb * ref).sum().item()
+    assert abs(dot.item() - d_ref) <= 1e-12 * abs(d_ref)
+    too_many_rows = 2 ** 31 - nnz                     # rows + non-zeros would no longer fit
+    with pytest.raises(RuntimeError, match="2\\^31"):
+        given["num_rows"] = too_many_rows
+        given["row_end_offsets"] = torch.zeros(too_many_rows + 1, device=dev, dtype=torch.int32)
+        ext.merged_spmv_launch(*[given[k] for k in ext.param_names()])
+
+
 def test_rmat_scale_22_against_the_library_product():
     w = W.rmat_spmv(22)
     ext = load_named(w.graph, build_if_missing=False)
