@@ -160,8 +160,8 @@ inline int grid_for_tiles(int num_tiles) {
 // ----------------------------------------------------------------------------------------------
 template <class G, int BLOCK, int IPT>
 __global__ void __launch_bounds__(BLOCK)
-reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const int num_rows, const int nnz,
-              const int2* __restrict__ coords, const int num_tiles, int* __restrict__ carry_row,
+reduce_kernel(const int2* __restrict__ coords, const int num_tiles, const int num_rows, const int* __restrict__ row_end,
+              const int nnz, const typename G::Params p, int* __restrict__ carry_row,
               typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials) {
   using V = typename G::Value;
   constexpr int TILE = BLOCK * IPT;
@@ -198,6 +198,12 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
 
+#ifdef FLEX_TUNE_COORD_PREFETCH  // tuning switch: pull the table line a later block on this XCD will need into L2
+  // (a vector load - a scalar one would return with the block's own coordinates - whose value is consumed
+  // after the vote barrier, so its register stays allocated while it is in flight)
+  const int coord_prefetch =
+      reinterpret_cast<const int*>(coords)[2 * min(tile + FLEX_TUNE_COORD_PREFETCH, num_tiles) + (tid & 1)];
+#endif
   const int2 c0 = coords[tile];
   const int2 c1 = coords[tile + 1];
   const int x0 = c0.x, y0 = c0.y;
@@ -289,6 +295,9 @@ reduce_kernel(const typename G::Params p, const int* __restrict__ row_end, const
   const unsigned long long wave_votes = __builtin_amdgcn_ballot_w64(my_vote);
   if (lane == 0) s_vote[wave] = (wave_votes != 0ull) ? 1 : 0;
   __syncthreads();
+#ifdef FLEX_TUNE_COORD_PREFETCH
+  asm volatile("" ::"v"(coord_prefetch));
+#endif
   int any_vote = 0;
 #pragma unroll
   for (int w = 0; w < NW; ++w) any_vote |= s_vote[w];

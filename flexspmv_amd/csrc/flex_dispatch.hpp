@@ -147,7 +147,7 @@ struct Dispatch {
       }
       if (timed) (void)hipEventRecord(g_timer.start, stream);
       hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid_for_tiles(l.num_tiles)), dim3(BLOCK), 0, stream,
-                         p, row_end, num_rows, nnz, (const int2*)coords, l.num_tiles, carry_row, carry_val, partials);
+                         (const int2*)coords, l.num_tiles, num_rows, row_end, nnz, p, carry_row, carry_val, partials);
       if (timed) g_timer.armed = (hipEventRecord(g_timer.stop, stream) == hipSuccess);
       V* block_partials = (V*)(ws + l.off_block_partials);
       hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, BLOCK / WAVE>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0, stream, p,
