@@ -166,6 +166,50 @@ def cpu_leg(w, result, outs, cpu_runs):
     return result
 
 
+def time_edge_list_preparation(w, steps):
+    """The step in front of a launch, on this workload's edge list: ascending COO row ids -> row pointer, the
+    stable sort by row of the shuffled list, and the permutation of one per-edge value array.  Bytes are
+    algorithmic: ids read once, pointer written once; for the permutation index + value read, value written."""
+    import torch
+    from flexspmv_amd import formats
+    ptr = torch.from_numpy(w.row_end_offsets).cuda()
+    rows = torch.repeat_interleave(torch.arange(w.num_rows, device="cuda", dtype=torch.int32),
+                                   (ptr[1:] - ptr[:-1]).to(torch.int64))
+    ne, nr = rows.numel(), w.num_rows
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            e1.synchronize()
+            best = min(best, e0.elapsed_time(e1) / reps)
+        return best
+
+    out = {}
+    ms = timed(lambda: formats.coo_rows_to_csr_async(rows, nr), steps)
+    got, findings = formats.coo_rows_to_csr_async(rows, nr)
+    ok = bool(torch.equal(got, ptr.to(torch.int32))) and int(findings[0]) == 0
+    b = 4 * ne + 4 * (nr + 1)
+    out["coo_rows_to_csr"] = {"ms": ms, "algorithmic_bytes": b, "gbs": b / ms / 1e6, "frac_of_hbm_peak":
+                              b / ms / 1e6 / HBM_PEAK_GBS, "matches_generator": ok}
+    shuffled = rows[torch.randperm(ne, device="cuda")]
+    ms = timed(lambda: formats.sort_edges_by_row(shuffled, nr), max(1, steps // 10))
+    out["sort_edges_by_row"] = {"ms": ms, "edges_per_s": ne / ms * 1e3}
+    _, perm = formats.sort_edges_by_row(shuffled, nr)
+    vals = torch.from_numpy(next(v for v in w.tensors.values() if v.dtype.kind == "f" and v.shape[0] == ne)).cuda()
+    dst = torch.empty_like(vals)
+    ms = timed(lambda: formats.gather_rows(vals, perm, out=dst), max(1, steps // 5))
+    b = ne * (4 + 2 * vals.element_size() * (vals.numel() // ne))
+    out["gather_rows"] = {"ms": ms, "algorithmic_bytes": b, "gbs": b / ms / 1e6, "order": "random permutation"}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -181,6 +225,8 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain elementwise copies (dst = src + 1) of 1 GiB, a kernel of known "
                          "traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--formats", action="store_true",
+                    help="also time the edge-list preparation kernels on this workload's edge list (extra JSON key)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists for it)",
@@ -273,6 +319,8 @@ def main() -> int:
                                 "parity_tolerance": c["tolerance"], "parity_ok": c["parity_ok"]}
     if others:
         line["other_workloads"] = others
+    if a.formats:
+        line["edge_list_preparation"] = time_edge_list_preparation(w, a.steps)
     print(json.dumps(line))
     return 0
 

@@ -49,10 +49,11 @@ def hipcc_path() -> str:
 
 
 def _csrc_digest() -> str:
+    """Digest of the headers a generated library is built from."""
     h = hashlib.sha1()
     for root in (CSRC_DIR, INCLUDE_DIR):
         for fn in sorted(os.listdir(root)):
-            if fn.endswith((".hpp", ".h")):
+            if fn.endswith((".hpp", ".h")) and fn != "flexspmv_formats.h":
                 with open(os.path.join(root, fn), "rb") as f:
                     h.update(fn.encode())
                     h.update(f.read())
@@ -125,3 +126,40 @@ def compile_many(graphs: Iterable[FusedGraphIR], jobs: int = 8, force: bool = Fa
     graphs = list(graphs)
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(graphs) or 1))) as pool:
         return list(pool.map(lambda g: compile_graph(g, force=force), graphs))
+
+
+# ---------------------------------------------------------------------------------------------
+# the edge-list preparation library (one per package, not per sub-graph)
+# ---------------------------------------------------------------------------------------------
+FORMATS_SOURCE = os.path.join(CSRC_DIR, "flex_formats.hip")
+FORMATS_LIBRARY = os.path.join(GENERATED_DIR, "libflexspmv_formats.so")
+
+
+def _formats_stamp() -> str:
+    h = hashlib.sha1()
+    for path in (FORMATS_SOURCE, os.path.join(INCLUDE_DIR, "flexspmv_formats.h")):
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest() + ":" + " ".join(HIPCC_FLAGS)
+
+
+def formats_is_current() -> bool:
+    stamp = _stamp_path(FORMATS_LIBRARY)
+    if not (os.path.exists(FORMATS_LIBRARY) and os.path.exists(stamp)):
+        return False
+    with open(stamp) as f:
+        return f.read() == _formats_stamp()
+
+
+def compile_formats(force: bool = False) -> str:
+    """Compile csrc/flex_formats.hip into _generated/libflexspmv_formats.so; returns its path."""
+    if not force and formats_is_current():
+        return FORMATS_LIBRARY
+    os.makedirs(GENERATED_DIR, exist_ok=True)
+    cmd = [hipcc_path(), *HIPCC_FLAGS, f"-I{INCLUDE_DIR}", FORMATS_SOURCE, "-o", FORMATS_LIBRARY]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise BuildError(f"hipcc failed for the formats library:\n{' '.join(cmd)}\n{proc.stdout}")
+    with open(_stamp_path(FORMATS_LIBRARY), "w") as f:
+        f.write(_formats_stamp())
+    return FORMATS_LIBRARY

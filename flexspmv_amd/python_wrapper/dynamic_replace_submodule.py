@@ -26,7 +26,9 @@ from typing import Dict, Iterable, List, Optional, Tuple
 import torch
 import torch.nn as nn
 
+from .. import formats as _formats
 from ..frontend.lite import Reducer, Selector
+from .edge_order import gather_edges, scatter_edges, stable_sort_by_row
 
 
 def get_submodules_wrapper(eqn, node_name, run_to_collect=True):
@@ -43,11 +45,13 @@ def get_submodules_wrapper(eqn, node_name, run_to_collect=True):
 
 def _coo_rows_to_csr_ptr(row_ids: torch.Tensor, num_rows: Optional[int] = None) -> Tuple[torch.Tensor, int]:
     """Sorted COO row ids -> CSR row pointer of length ``num_rows + 1`` (int64, device of ``row_ids``)."""
-    row_ids = row_ids.to(torch.int64)
     if num_rows is None:
         if row_ids.numel() == 0:
             raise RuntimeError("row_ids is empty; cannot infer num_rows")
         num_rows = int(row_ids.max().item()) + 1
+    if row_ids.is_cuda:     # the package's own kernel; the reference's int64 result type is kept
+        return _formats.coo_rows_to_csr(row_ids, num_rows).to(torch.int64), num_rows
+    row_ids = row_ids.to(torch.int64)
     if row_ids.numel() > 1 and bool((row_ids[1:] < row_ids[:-1]).any()):
         raise RuntimeError("Reducer row ids must be sorted ascending for the CSR conversion; sort the edges "
                            "by destination row first (flexspmv_amd.python_wrapper.edge_order)")
@@ -199,8 +203,11 @@ class _DynamicCudaWrapper(nn.Module):
         perm = None
         if self.edge_permutation is not None:
             perm = self._on("edge_permutation", device)
+            if perm.is_cuda and perm.dtype != torch.int32:      # the permutation kernels take int32
+                perm = perm.to(torch.int32)
+                self.edge_permutation = perm
             for n in self._non_gather_value_inputs:
-                arg_map[n] = arg_map[n].index_select(0, perm)
+                arg_map[n] = gather_edges(arg_map[n], perm)
         call_args = [arg_map[n] for n in self._non_gather_value_inputs]
         call_args += [arg_map[n] for n in self._gather_value_inputs]
         call_args += [self._on(b, device) for b in self._selector_buf_names]
@@ -210,12 +217,12 @@ class _DynamicCudaWrapper(nn.Module):
         if perm is not None:            # per-edge stores went to the sorted copies: put them back
             for n, a in zip(self._input_param_names, args):
                 if n in self._written_inputs and n in self._non_gather_value_inputs:
-                    a.index_copy_(0, perm, arg_map[n].view((a.shape[0],) + tuple(a.shape[1:])))
+                    scatter_edges(arg_map[n], perm, out=a)
         if outs is None:
             return []
         outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]
         if perm is not None and self._per_edge_outputs is not None:
-            outs = [torch.empty_like(o).index_copy_(0, perm, o) if per_edge else o
+            outs = [scatter_edges(o, perm) if per_edge else o
                     for o, per_edge in zip(outs, self._per_edge_outputs)]
         if self._output_shapes is not None and len(self._output_shapes) == len(outs):
             outs = [o.view(s) if s and o.numel() == _numel(s) else o for o, s in zip(outs, self._output_shapes)]
@@ -236,11 +243,20 @@ def build_wrapper(gm, ext) -> _DynamicCudaWrapper:
     selector_idx_tensors = [mod.idx for _, mod in selector_modules]
     edge_permutation = None
     if reducer_mod is not None:
-        row_ids = reducer_mod.idx.to(torch.int64)
-        if row_ids.numel() > 1 and bool((row_ids[1:] < row_ids[:-1]).any()):
-            row_ids, edge_permutation = torch.sort(row_ids, stable=True)
-            selector_idx_tensors = [t.index_select(0, edge_permutation.to(t.device)) for t in selector_idx_tensors]
-        row_end_offsets, _ = _coo_rows_to_csr_ptr(row_ids, int(reducer_mod.n))
+        row_ids, num_rows = reducer_mod.idx, int(reducer_mod.n)
+        if row_ids.is_cuda:         # one pass answers "ascending?" and, if so, already is the row pointer
+            row_end_offsets, findings = _formats.coo_rows_to_csr_async(row_ids, num_rows)
+            found = int(findings[0])
+            if found & _formats.FINDING_OUT_OF_RANGE:
+                raise RuntimeError("Reducer row ids outside [0, num_rows)")
+            unsorted = bool(found & _formats.FINDING_UNSORTED)
+        else:
+            unsorted = row_ids.numel() > 1 and bool((row_ids[1:] < row_ids[:-1]).any())
+        if unsorted:
+            row_ids, edge_permutation = stable_sort_by_row(row_ids, num_rows)
+            selector_idx_tensors = [gather_edges(t, edge_permutation) for t in selector_idx_tensors]
+        if unsorted or not row_ids.is_cuda:
+            row_end_offsets, _ = _coo_rows_to_csr_ptr(row_ids, num_rows)
     else:
         row_end_offsets = None
     gather_value_inputs = _infer_gather_value_inputs(gm, [q for q, _ in selector_modules])

@@ -2,14 +2,43 @@
 
 The reference converts the Reducer's COO row ids with ``torch._convert_indices_from_coo_to_csr``
 (python_wrapper/dynamic_replace_submodule.py:20-41), which is only meaningful when the ids are already
-sorted.  These helpers produce that order on the device the ids live on (torch's sort is a device radix
-sort), once, at model set-up time.
+sorted.  These helpers produce that order, once, at model set-up time.  Tensors on the GPU go through the
+package's own kernels (``flexspmv_amd.formats``: radix sort by row, row pointer from the ids, permutation
+of per-edge tensors); tensors in host memory, which only model set-up on a machine without a GPU sees, go
+through the equivalent torch calls.
 """
 from __future__ import annotations
 
 from typing import Sequence, Tuple
 
 import torch
+
+from .. import formats
+
+
+def stable_sort_by_row(row_ids: torch.Tensor, num_rows: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(sorted ids, permutation)``; on the GPU both are int32, in host memory int64."""
+    if row_ids.is_cuda:
+        return formats.sort_edges_by_row(row_ids, num_rows)
+    return torch.sort(row_ids.to(torch.int64), stable=True)
+
+
+def gather_edges(t: torch.Tensor, permutation: torch.Tensor) -> torch.Tensor:
+    """``t[permutation]`` along the leading dimension, contiguous."""
+    if t.is_cuda and t.element_size() * (t.numel() // max(t.shape[0], 1)) % 4 == 0 and t.shape[0] > 0:
+        return formats.gather_rows(t, permutation.to(device=t.device, dtype=torch.int32))
+    return t.index_select(0, permutation.to(device=t.device, dtype=torch.int64)).contiguous()
+
+
+def scatter_edges(src: torch.Tensor, permutation: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+    """``out[permutation[k]] = src[k]`` along the leading dimension (``out`` is created when not given)."""
+    if out is None:
+        out = torch.empty_like(src, memory_format=torch.contiguous_format)
+    if (src.is_cuda and out.is_contiguous() and src.shape[0] > 0
+            and src.element_size() * (src.numel() // src.shape[0]) % 4 == 0):
+        return formats.scatter_rows(src.reshape(out.shape), permutation.to(device=src.device, dtype=torch.int32),
+                                    out=out)
+    return out.index_copy_(0, permutation.to(device=src.device, dtype=torch.int64), src.reshape(out.shape))
 
 
 def sort_edges_by_row(row_ids: torch.Tensor, *edge_tensors: torch.Tensor) -> Tuple[torch.Tensor, ...]:
@@ -20,13 +49,14 @@ def sort_edges_by_row(row_ids: torch.Tensor, *edge_tensors: torch.Tensor) -> Tup
     order of the original edge list is preserved."""
     if row_ids.dim() != 1:
         raise ValueError("row_ids must be 1-D")
-    sorted_ids, perm = torch.sort(row_ids, stable=True)
+    num_rows = int(row_ids.max()) + 1 if row_ids.numel() else 1
+    sorted_ids, perm = stable_sort_by_row(row_ids, num_rows)
     moved = []
     for t in edge_tensors:
         if t.shape[0] != row_ids.shape[0]:
             raise ValueError("every edge tensor must have one leading entry per edge")
-        moved.append(t.index_select(0, perm).contiguous())
-    return (sorted_ids, perm, *moved)
+        moved.append(gather_edges(t, perm))
+    return (sorted_ids.to(row_ids.dtype), perm.to(torch.int64), *moved)
 
 
 def half_edges(src: torch.Tensor, dst: torch.Tensor, *edge_tensors: torch.Tensor) -> Tuple[torch.Tensor, ...]:
@@ -47,7 +77,16 @@ def half_edges(src: torch.Tensor, dst: torch.Tensor, *edge_tensors: torch.Tensor
 
 
 def coo_to_csr(row_ids: torch.Tensor, num_rows: int) -> torch.Tensor:
-    """int32 CSR row pointer of sorted row ids (histogram + inclusive scan on the ids' device)."""
+    """int32 CSR row pointer of sorted row ids."""
+    if row_ids.is_cuda:
+        try:
+            return formats.coo_rows_to_csr(row_ids, num_rows)
+        except RuntimeError as e:
+            if "sorted" in str(e):
+                raise ValueError("row ids are not sorted; use sort_edges_by_row first") from e
+            if "outside" in str(e):
+                raise ValueError("row ids outside [0, num_rows)") from e
+            raise
     if row_ids.numel() > 1 and bool((row_ids[1:] < row_ids[:-1]).any()):
         raise ValueError("row ids are not sorted; use sort_edges_by_row first")
     counts = torch.bincount(row_ids.to(torch.int64), minlength=num_rows)
