@@ -277,3 +277,42 @@ def test_sort_at_benchmark_size_is_a_stable_permutation():
     same_row = sorted_rows[1:] == sorted_rows[:-1]
     assert bool((perm[1:][same_row] > perm[:-1][same_row]).all())               # stable
     assert torch.equal(formats.coo_rows_to_csr(sorted_rows, w.num_rows), ptr.to(torch.int32))
+
+
+@pytest.mark.gpu
+def test_row_pointer_and_permutation_replay_in_a_hip_graph():
+    """The row-pointer call and the permutation calls are captured once and replayed on new contents of
+    the same buffers (eager work and synchronisation between the replays); every replay equals the eager result."""
+    torch = _cuda()
+    rng = np.random.default_rng(31)
+    num_rows, ne = 30_000, 120_000
+    ids = torch.zeros(ne, dtype=torch.int32, device="cuda")
+    vals = torch.zeros(ne, 2, dtype=torch.float64, device="cuda")
+    perm = torch.from_numpy(rng.permutation(ne).astype(np.int32)).cuda()
+    ids.copy_(torch.from_numpy(_edge_list(rng, num_rows, ne, "uniform").astype(np.int32)))
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        for _ in range(2):
+            formats.coo_rows_to_csr_async(ids, num_rows)
+            formats.scatter_rows(formats.gather_rows(vals, perm), perm)
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_ptr, g_findings = formats.coo_rows_to_csr_async(ids, num_rows)
+        g_moved = formats.gather_rows(vals, perm)
+        g_back = formats.scatter_rows(g_moved, perm)
+    for rep, kind in enumerate(["skewed", "few_rows", "uniform", "tail"]):
+        rows = _edge_list(rng, num_rows, ne, kind)
+        v = rng.standard_normal((ne, 2))
+        ids.copy_(torch.from_numpy(rows.astype(np.int32)))
+        vals.copy_(torch.from_numpy(v))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(g_findings[0]) == 0
+        assert np.array_equal(g_ptr.cpu().numpy(), FO.coo_rows_to_csr(rows, num_rows)), (rep, kind)
+        assert np.array_equal(g_moved.cpu().numpy(), FO.gather_rows(v, perm.cpu().numpy()))
+        assert torch.equal(g_back, vals)
+        eager_ptr = formats.coo_rows_to_csr(ids, num_rows)          # eager work between replays
+        assert torch.equal(eager_ptr, g_ptr)
