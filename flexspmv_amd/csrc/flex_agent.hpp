@@ -159,10 +159,10 @@ inline int grid_for_tiles(int num_tiles) {
 // the tile's open last row becomes a carry record for fixup_kernel.
 // ----------------------------------------------------------------------------------------------
 template <class G, int BLOCK, int IPT>
-__global__ void __launch_bounds__(BLOCK)
-reduce_kernel(const int2* __restrict__ coords, const int num_tiles, const int num_rows, const int* __restrict__ row_end,
-              const int nnz, const typename G::Params p, int* __restrict__ carry_row,
-              typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials) {
+__device__ __forceinline__ void
+reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, const int* __restrict__ row_end,
+            const int nnz, const typename G::Params& p, int* __restrict__ carry_row,
+            typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials) {
   using V = typename G::Value;
   constexpr int TILE = BLOCK * IPT;
   constexpr int NW = BLOCK / WAVE;
@@ -192,20 +192,10 @@ reduce_kernel(const int2* __restrict__ coords, const int num_tiles, const int nu
   __shared__ int s_wave_key[NW];
   __shared__ V s_wave_val[NW][REDN];
 
-  const int tile = tile_of_block(blockIdx.x, num_tiles);
-  if (tile >= num_tiles) return;
   const int tid = threadIdx.x;
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
 
-#ifdef FLEX_TUNE_COORD_PREFETCH  // tuning switch: pull the table line a later block on this XCD will need into L2
-  // (a vector load - a scalar one would return with the block's own coordinates - whose value is consumed
-  // after the vote barrier, so its register stays allocated while it is in flight)
-  const int coord_prefetch =
-      reinterpret_cast<const int*>(coords)[2 * min(tile + FLEX_TUNE_COORD_PREFETCH, num_tiles) + (tid & 1)];
-#endif
-  const int2 c0 = coords[tile];
-  const int2 c1 = coords[tile + 1];
   const int x0 = c0.x, y0 = c0.y;
   const int R = c1.x - c0.x;  // row ends inside this tile
   const int Z = c1.y - c0.y;  // non-zeros inside this tile
@@ -295,9 +285,6 @@ reduce_kernel(const int2* __restrict__ coords, const int num_tiles, const int nu
   const unsigned long long wave_votes = __builtin_amdgcn_ballot_w64(my_vote);
   if (lane == 0) s_vote[wave] = (wave_votes != 0ull) ? 1 : 0;
   __syncthreads();
-#ifdef FLEX_TUNE_COORD_PREFETCH
-  asm volatile("" ::"v"(coord_prefetch));
-#endif
   int any_vote = 0;
 #pragma unroll
   for (int w = 0; w < NW; ++w) any_vote |= s_vote[w];
@@ -518,6 +505,41 @@ reduce_kernel(const int2* __restrict__ coords, const int num_tiles, const int nu
       for (int c = 0; c < AGG; ++c) agg_partials[((size_t)tile * NW + wave) * AGG + c] = agg.v[c];
     }
   }
+}
+
+// One block per tile by default.  With FLEX_TUNE_PERSISTENT (tuning switch) a launch has at most that many
+// blocks per CU; each walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... and reads the coordinates of its next
+// tile while it works on the current one.
+template <class G, int BLOCK, int IPT>
+__global__ void __launch_bounds__(BLOCK)
+reduce_kernel(const int2* __restrict__ coords, const int num_tiles, const int num_rows, const int* __restrict__ row_end,
+              const int nnz, const typename G::Params p, int* __restrict__ carry_row,
+              typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials) {
+#ifdef FLEX_TUNE_PERSISTENT
+  int tile = blockIdx.x;
+  if (tile >= num_tiles) return;
+  int2 c0 = coords[tile], c1 = coords[tile + 1];
+  while (true) {
+    const int next = tile + (int)gridDim.x;
+    const bool more = next < num_tiles;
+    int2 n0 = c0, n1 = c1;
+    if (more) {
+      n0 = coords[next];
+      n1 = coords[next + 1];
+    }
+    reduce_tile<G, BLOCK, IPT>(tile, c0, c1, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
+    if (!more) break;
+    __syncthreads();  // the tile's LDS is free again
+    tile = next;
+    c0 = n0;
+    c1 = n1;
+  }
+#else
+  const int tile = tile_of_block(blockIdx.x, num_tiles);
+  if (tile >= num_tiles) return;
+  reduce_tile<G, BLOCK, IPT>(tile, coords[tile], coords[tile + 1], num_rows, row_end, nnz, p, carry_row, carry_val,
+                             agg_partials);
+#endif
 }
 
 // ----------------------------------------------------------------------------------------------

@@ -146,7 +146,12 @@ struct Dispatch {
                            row_end, num_rows, nnz, coords);
       }
       if (timed) (void)hipEventRecord(g_timer.start, stream);
-      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(grid_for_tiles(l.num_tiles)), dim3(BLOCK), 0, stream,
+#ifdef FLEX_TUNE_PERSISTENT
+      const int reduce_grid = l.num_tiles < 256 * FLEX_TUNE_PERSISTENT ? l.num_tiles : 256 * FLEX_TUNE_PERSISTENT;
+#else
+      const int reduce_grid = grid_for_tiles(l.num_tiles);
+#endif
+      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(reduce_grid), dim3(BLOCK), 0, stream,
                          (const int2*)coords, l.num_tiles, num_rows, row_end, nnz, p, carry_row, carry_val, partials);
       if (timed) g_timer.armed = (hipEventRecord(g_timer.stop, stream) == hipSuccess);
       V* block_partials = (V*)(ws + l.off_block_partials);
