@@ -81,8 +81,10 @@ def main(argv=None) -> int:
     ap.add_argument("--points", type=int, default=None, help="mesh points of the shallow-water model")
     ap.add_argument("--n", type=int, default=None, help="lattice edge of the spring-mass model")
     ap.add_argument("--dt", type=float, default=None, help="time step of the shallow-water model")
+    ap.add_argument("--mesh", default=None, help="shallow-water model: read the mesh from this .npz / .hdf5 file "
+                                                 "(shallow_water.save_mesh writes one)")
     a = ap.parse_args(argv)
-    kw = {k: v for k, v in (("points", a.points), ("n", a.n), ("dt", a.dt)) if v is not None}
+    kw = {k: v for k, v in (("points", a.points), ("n", a.n), ("dt", a.dt), ("mesh", a.mesh)) if v is not None}
 
     def sync():
         if a.device.startswith("cuda"):

@@ -17,10 +17,13 @@ def _system(device="cpu", dtype=torch.float64, num_nnz=64, sorted_rows=True):
     return make_system(num_nnz, 17, 13, device=device, dtype=dtype, sorted_rows=sorted_rows)
 
 
-def _swe(device="cpu", dtype=torch.float64, points=900, dt=0.0005):
+def _swe(device="cpu", dtype=torch.float64, points=900, dt=0.0005, mesh=None):
     """``dt`` is a literal of the generated kernels (as every Python number of a model is): another value
-    means other libraries.  0.0005 is stable up to about 250k mesh points (gravity wave speed is ~1)."""
-    from .shallow_water import ShallowWaterEquation, synthetic_mesh
+    means other libraries.  0.0005 is stable up to about 250k mesh points (gravity wave speed is ~1).
+    ``mesh``: a file written by ``shallow_water.save_mesh`` instead of a generated mesh."""
+    from .shallow_water import ShallowWaterEquation, load_mesh, synthetic_mesh
+    if mesh is not None:
+        return ShallowWaterEquation(load_mesh(mesh, dtype=dtype, device=device), dt=dt)
     return ShallowWaterEquation(synthetic_mesh(points, dtype=dtype, device=device), dt=dt)
 
 

@@ -5,7 +5,9 @@ cell-centred height ``h`` and momenta ``uh, vh``; every interior face is a direc
 ``src -> dst`` sorted by ``dst``; face values are interpolated with weight ``alpha``; fluxes through the
 scaled face normals ``(sx, sy)`` are summed per destination cell by one ``Reducer``; wall faces add the
 pressure term through a second ``Reducer`` over the boundary cells.  The reference reads its mesh from
-HDF5 files; here the same arrays come from a Delaunay triangulation of a jittered lattice of points."""
+HDF5 files; here the same arrays come from a Delaunay triangulation of a jittered lattice of points, or from
+a file written by ``save_mesh`` (``.npz`` everywhere, ``.hdf5`` where h5py exists) and read dataset by
+dataset like the reference's."""
 from __future__ import annotations
 
 from typing import Dict
@@ -71,6 +73,35 @@ def synthetic_mesh(points: int = 2000, seed: int = 3, dtype=torch.float64, devic
             "x": val(centroid[:, 0]), "y": val(centroid[:, 1]), "area": val(area),
             "sx": val(n_in[:, 0]), "sy": val(n_in[:, 1]), "bsx": val(n_b[:, 0]), "bsy": val(n_b[:, 1]),
             "alpha": val(alpha), "h": val(h0)}
+
+
+MESH_INDEX_ARRAYS = ("src", "dst", "bcells")
+MESH_VALUE_ARRAYS = ("x", "y", "area", "sx", "sy", "bsx", "bsy", "alpha", "h")
+
+
+def save_mesh(mesh: Dict[str, torch.Tensor], path: str) -> None:
+    """Write the arrays of ``synthetic_mesh`` (or any mesh with the same names) to ``path``."""
+    esr.save_arrays(path, {k: mesh[k] for k in MESH_INDEX_ARRAYS + MESH_VALUE_ARRAYS + ("nc",)})
+
+
+def load_mesh(path: str, dtype=torch.float64, device="cpu") -> Dict[str, torch.Tensor]:
+    """The mesh dict of a file, read one dataset at a time (the reference's ``esr.hdf5(path, name, dtype=...)``
+    calls, swe_main.py:19-71); ``nc`` is taken from the file or, failing that, from the cell arrays."""
+    mesh: Dict[str, torch.Tensor] = {}
+    for name in MESH_INDEX_ARRAYS:
+        mesh[name] = esr.hdf5(path, name, dtype=torch.long, device=device)
+    for name in MESH_VALUE_ARRAYS:
+        mesh[name] = esr.hdf5(path, name, dtype=dtype, device=device)
+    mesh["nc"] = int(esr.hdf5(path, "nc")) if "nc" in esr.datasets(path) else int(mesh["x"].shape[0])
+    ne, nb = mesh["src"].shape[0], mesh["bcells"].shape[0]
+    for name, n in (("dst", ne), ("sx", ne), ("sy", ne), ("alpha", ne), ("bsx", nb), ("bsy", nb),
+                    ("y", mesh["nc"]), ("area", mesh["nc"]), ("h", mesh["nc"]), ("x", mesh["nc"])):
+        if mesh[name].shape[0] != n:
+            raise ValueError(f"{path}: array {name!r} has {mesh[name].shape[0]} entries, expected {n}")
+    for name in MESH_INDEX_ARRAYS:
+        if mesh[name].numel() and (int(mesh[name].min()) < 0 or int(mesh[name].max()) >= mesh["nc"]):
+            raise ValueError(f"{path}: {name!r} refers to cells outside [0, {mesh['nc']})")
+    return mesh
 
 
 class ShallowWaterEquation(esr.Module):

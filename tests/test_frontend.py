@@ -541,3 +541,57 @@ def test_tensor_names_that_look_like_kernel_internals_and_a_gathered_output():
         GraphBuilder("bad").placeholder("q_e")
     with pytest.raises(ValueError, match="not usable"):
         GraphBuilder("bad").placeholder("double")
+
+
+# ---------------------------------------------------------------------------------------------
+# named arrays from files (the esr.hdf5 stand-in)
+# ---------------------------------------------------------------------------------------------
+def test_mesh_file_round_trip_gives_the_same_model(tmp_path):
+    from flexspmv_amd.drivers.shallow_water import ShallowWaterEquation, load_mesh, save_mesh, synthetic_mesh
+    mesh = synthetic_mesh(400, seed=5)
+    path = str(tmp_path / "mesh.npz")
+    save_mesh(mesh, path)
+    assert set(esr.datasets(path)) >= {"src", "dst", "bcells", "x", "h", "nc"}
+    assert esr.hdf5(path, "src", dtype=torch.long).dtype == torch.int64
+    assert esr.hdf5(path, "h", dtype=torch.float32).dtype == torch.float32
+    loaded = load_mesh(path)
+    for k, v in mesh.items():
+        assert (loaded[k] == v) if k == "nc" else torch.equal(loaded[k], v), k
+    a, b = ShallowWaterEquation(mesh, dt=0.0005), ShallowWaterEquation(loaded, dt=0.0005)
+    for _ in range(3):
+        a()
+        b()
+    assert torch.equal(a.h, b.h) and torch.equal(a.uh, b.uh)
+
+
+def test_array_files_fail_loudly(tmp_path):
+    import numpy as np
+    path = str(tmp_path / "arrays.npz")
+    esr.save_arrays(path, {"a": torch.arange(4), "b": np.ones((2, 2)), "n": 3})
+    assert esr.hdf5(path, "a").tolist() == [0, 1, 2, 3] and int(esr.hdf5(path, "n")) == 3
+    with pytest.raises(KeyError, match="no array 'c'"):
+        esr.hdf5(path, "c")
+    with pytest.raises(FileNotFoundError):
+        esr.hdf5(str(tmp_path / "missing.npz"), "a")
+    with pytest.raises(RuntimeError, match="unknown container"):
+        esr.save_arrays(str(tmp_path / "arrays.bin"), {"a": torch.arange(4)})
+    h5 = str(tmp_path / "mesh.hdf5")
+    try:
+        import h5py  # noqa: F401
+    except ImportError:
+        open(h5, "wb").close()
+        with pytest.raises(RuntimeError, match="h5py"):
+            esr.hdf5(h5, "src")
+        with pytest.raises(RuntimeError, match="h5py"):
+            esr.save_arrays(h5, {"a": torch.arange(4)})
+    else:
+        esr.save_arrays(h5, {"a": torch.arange(4)})
+        assert esr.hdf5(h5, "a").tolist() == [0, 1, 2, 3]
+    from flexspmv_amd.drivers.shallow_water import load_mesh, save_mesh, synthetic_mesh
+    mesh = synthetic_mesh(100, seed=1)
+    mesh["src"] = mesh["src"].clone()
+    mesh["src"][0] = mesh["nc"]              # a face that refers to a cell that does not exist
+    bad = str(tmp_path / "bad.npz")
+    save_mesh(mesh, bad)
+    with pytest.raises(ValueError, match="outside"):
+        load_mesh(bad)
