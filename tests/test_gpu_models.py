@@ -146,6 +146,35 @@ def test_graph_replay_of_a_model_step_matches_eager_launches():
     assert float(scratch[0]) == steps
 
 
+def test_graph_replay_with_an_unordered_edge_list():
+    """The toy model with row ids in random order: the per-step permutation of the streamed edge tensors is
+    part of the captured graph; replays equal eager steps bit for bit."""
+    from flexspmv_amd.python_wrapper.graph_replay import capture_step
+    print("case graph replay system unsorted", flush=True)
+    steps = 4
+
+    def build():
+        model = MODELS["system"](device="cuda", num_nnz=20000, sorted_rows=False)
+        [compiled] = esr.compile([model], "torch")
+        report = accelerate(compiled, prefix="system", build_if_missing=False)
+        assert all(v == "replaced" for v in report.values()), report
+        return compiled
+
+    eager = build()
+    for _ in range(2 + steps):
+        eager()
+    torch.cuda.synchronize()
+    want = ab_check.save_state(eager)
+    replayed = build()
+    replay = capture_step(replayed, warmup=2)
+    for i in range(steps):
+        replay()
+        torch.cuda.synchronize()
+    got = ab_check.save_state(replayed)
+    for k in want:
+        assert torch.equal(want[k], got[k]), k
+
+
 def test_conjugate_gradients_on_the_fused_poisson_operator():
     """The solver loop around the fused ``A p`` / ``p . A p`` launch converges to the solution of a
     manufactured problem, and launches after the first reuse the tile table."""
