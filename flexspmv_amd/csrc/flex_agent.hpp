@@ -289,7 +289,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
 #pragma unroll
   for (int w = 0; w < NW; ++w) any_vote |= s_vote[w];
 #ifdef FLEX_TUNE_FORCE_MERGE  // tuning switch: always the merge path, decided at run time (same code)
-  const bool irregular = any_vote != 0 || num_tiles > 0;
+  const bool irregular = any_vote != 0 || nnz > 0;
 #else
   const bool irregular = any_vote != 0;
 #endif
