@@ -9,8 +9,9 @@ torch's current stream.  Differences from the reference, on purpose:
 
 * outputs are ``torch.empty`` - the kernels write every element exactly once, so the reference's
   ``torch::zeros`` fill (codegen/merged_gen_binding.py:100-104) is unnecessary traffic;
-* scratch is a cached tensor per (library, device) instead of ``cudaMalloc`` / ``cudaFree`` per
-  call (cuda_template/merged_binding_template.cu:42-49);
+* scratch is a cached tensor per (library, device, stream) instead of ``cudaMalloc`` / ``cudaFree``
+  per call (cuda_template/merged_binding_template.cu:42-49): launches of one library on different
+  streams never share tile table, carries or partials, launches on one stream are ordered by it;
 * an unsupported dtype raises (the reference's CUDA binding only logs and falls off the function,
   :65-68; its CPU binding raises, cpu_template/merged_binding_template_cpu.cpp:45-46).
 
@@ -27,12 +28,13 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 from . import build as _build
 from .ir import FusedGraphIR
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 FLAG_TIME_KERNEL = 1
 FLAG_REUSE_TILES = 2
+FLAG_KEEP_TILES = 4
 DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
 EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
-                    "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms")
+                    "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms", "flexspmv_tiling")
 
 
 class LaunchArgs(ctypes.Structure):
@@ -81,6 +83,8 @@ def load_library(path: str) -> ctypes.CDLL:
     lib.flexspmv_last_kernel_ms.restype = ctypes.c_int
     lib.flexspmv_abi_version.argtypes = []
     lib.flexspmv_abi_version.restype = ctypes.c_int
+    lib.flexspmv_tiling.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_int32)]
+    lib.flexspmv_tiling.restype = ctypes.c_int
     if lib.flexspmv_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{path}: built for interface version {lib.flexspmv_abi_version()}, "
                            f"this package speaks {ABI_VERSION}")
@@ -104,18 +108,26 @@ class HipExtension:
         self._value_names: List[str] = list(self.signature["value_inputs"])
         self._index_names: List[str] = list(self.signature["index_inputs"])
         self._row_aligned = set(self.signature.get("row_aligned_index_inputs", []))
+        self._row_indexed = set(self.signature.get("row_indexed_value_inputs", []))
+        # debugging aid: compare every row-aligned index array with the row ids of row_end_offsets on each
+        # launch (a library that serves such a selector from the merge path never reads the array, so a
+        # caller who passes another index gets the rows' own items without an error otherwise)
+        self.verify_row_aligned = False
         self._outputs = self.signature["outputs"]
         self._has_reducer = bool(self.signature["has_reducer"])
         self._streamed = set(self.signature["non_gather_value_inputs"])
         self._dtypes = set(self.signature["dtypes"])
         self._param_names = [p["name"] for p in self.signature["params"]]
-        self._workspace: Dict[Any, Any] = {}
+        self._workspace: Dict[Any, Any] = {}   # (device index, stream handle) -> scratch tensor
+        self._captured = set()                 # keys whose buffer a stream capture has recorded
+        self._retained: List[Any] = []         # replaced buffers that a captured graph still refers to
         self.time_kernel = False   # set True to bracket the dominant kernel of each launch with events
         # Reuse of the tile table between launches on the same, unmodified row_end_offsets tensor (the
         # reference's wrapper keeps it as an immutable buffer, dynamic_replace_submodule.py:118-137).
         # Off by default: every launch then does all the work a launch of the reference does.
         self.reuse_tiles = False
         self._tile_key = None
+        self.extra_flags = 0       # FLAG_* bits added to every launch (FLAG_KEEP_TILES for debugging)
 
     # -- helpers -------------------------------------------------------------------------
     def param_names(self) -> List[str]:
@@ -136,13 +148,39 @@ class HipExtension:
     def workspace_bytes(self, dtype: str, num_rows: int, ne: int) -> int:
         return int(self._lib.flexspmv_workspace_bytes(DTYPE_CODES[dtype], num_rows, ne))
 
-    def _scratch(self, device, nbytes: int):
+    def _scratch(self, device, stream, nbytes: int):
+        """Scratch of this library for launches on ``stream`` of ``device``.
+
+        The buffer is allocated on that stream and only ever used on it, so when a larger launch replaces
+        it the caching allocator hands the old block out again in stream order - nothing still running
+        can see it change.  A buffer that a stream capture has recorded is kept for the life of the
+        library (a replayed graph keeps using its address), and growing during a capture is refused:
+        run the step once eagerly first, as capture_step does."""
         import torch
-        buf = self._workspace.get(device)
+        key = (device.index if device.index is not None else torch.cuda.current_device(), int(stream.cuda_stream))
+        capturing = torch.cuda.is_current_stream_capturing()
+        buf = self._workspace.get(key)
         if buf is None or buf.numel() < nbytes:
-            buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
-            self._workspace[device] = buf
+            _check(not capturing, "FlexSpmv scratch cannot grow during a stream capture: "
+                                  "launch once with these sizes before capturing")
+            if buf is not None and key in self._captured:
+                self._retained.append(buf)
+                self._captured.discard(key)
+            with torch.cuda.stream(stream):
+                buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+            self._workspace[key] = buf
+        if capturing:
+            self._captured.add(key)
         return buf
+
+    def workspace_of(self, device, stream=None):
+        """The scratch tensor of launches on ``stream`` (default: the current stream) of ``device``, or
+        None before the first such launch.  For debugging (the tile table sits at its start)."""
+        import torch
+        device = torch.device(device)
+        stream = stream if stream is not None else torch.cuda.current_stream(device)
+        index = device.index if device.index is not None else torch.cuda.current_device()
+        return self._workspace.get((index, int(stream.cuda_stream)))
 
     # -- the call ------------------------------------------------------------------------
     def merged_spmv_launch(self, *args, **kwargs):
@@ -181,6 +219,21 @@ class HipExtension:
                 _check(t.numel() >= ne * dims[n], f"{n} must hold one item of width {dims[n]} per edge ({ne})")
         if self._has_reducer:
             _check(ro.numel() == num_rows + 1, "row_end_offsets must have length num_rows + 1")
+            _check(num_rows + ne < 2 ** 31, "num_rows + ne must stay below 2^31 (32-bit offsets)")
+            # a source gathered through a row-aligned selector is read at every row id of a tile, empty
+            # rows included: a tensor shorter than num_rows would be read out of bounds
+            for n, t in zip(self._value_names, values):
+                if n in self._row_indexed:
+                    _check(t.numel() >= num_rows * dims[n],
+                           f"{n} must hold one item of width {dims[n]} per row ({num_rows}): it is gathered "
+                           f"through a selector declared equal to the reducer's row ids")
+            if self.verify_row_aligned and self._row_aligned:
+                row_ids = torch.repeat_interleave(torch.arange(num_rows, device=ro.device, dtype=torch.int32),
+                                                  (ro[1:] - ro[:-1]).to(torch.int64))
+                for n, t in zip(self._index_names, indices):
+                    if n in self._row_aligned:
+                        _check(bool(torch.equal(t, row_ids)), f"{n} was declared equal to the reducer's row ids "
+                                                              f"(row_aligned) but differs from them")
 
         device = dispatch.device
         outs = []
@@ -193,7 +246,8 @@ class HipExtension:
             outs.append(torch.empty(shape, dtype=dispatch.dtype, device=device))
 
         ws_bytes = self.workspace_bytes(dt, num_rows, ne)
-        ws = self._scratch(device, ws_bytes)
+        stream = torch.cuda.current_stream(device)
+        ws = self._scratch(device, stream, ws_bytes)
 
         def ptr_array(tensors):
             arr = (ctypes.c_void_p * max(len(tensors), 1))()
@@ -214,14 +268,14 @@ class HipExtension:
         la.row_end_offsets = ro.data_ptr()
         la.num_rows, la.num_cols, la.ne = num_rows, num_cols, ne
         la.workspace, la.workspace_bytes = ws.data_ptr(), ws.numel()
-        la.flags = FLAG_TIME_KERNEL if self.time_kernel else 0
+        la.flags = (FLAG_TIME_KERNEL if self.time_kernel else 0) | int(self.extra_flags)
         if self.reuse_tiles and self._has_reducer:
             key = (ro.data_ptr(), ro._version, num_rows, ne, dt, ws.data_ptr(), str(device))
             if key == self._tile_key:
                 la.flags |= FLAG_REUSE_TILES
             self._tile_key = key
         with torch.cuda.device(device):
-            la.stream = torch.cuda.current_stream(device).cuda_stream
+            la.stream = stream.cuda_stream
             rc = self._lib.flexspmv_launch(ctypes.byref(la))
         if rc != 0:
             raise RuntimeError(f"merged_spmv_launch failed ({rc}): {self._lib.flexspmv_last_error().decode()}")

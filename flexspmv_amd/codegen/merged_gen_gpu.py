@@ -31,6 +31,7 @@ VERBOSE_ENV = "EASIER_VERBOSE_CODEGEN"  # same switch as the reference (codegen/
 # (160 KiB LDS per CU on gfx950).
 LDS_BUDGET_BYTES = 36 * 1024
 BLOCK_THREADS = 256
+DEFAULT_XCD_RUN = 1
 
 
 @dataclass
@@ -282,7 +283,8 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
 
     ``dtypes`` lists the value types to instantiate (default float32 + float64, plus int64 when the
     dispatch input was traced as int64 - the reference's rule, codegen/merged_gen_binding.py:143-157).
-    ``policy`` may override ``block``, ``ipt_f32``, ``ipt_f64``.
+    ``policy`` may override ``block``, ``ipt_f32``, ``ipt_f64``, ``ipt_flat`` and ``xcd_run`` (consecutive
+    tiles handed to one XCD; 1 = round-robin).
     """
     inputs, outputs, selector_register, map_ops, red_ops, agg_ops = ir.six()
     kp = analyse(ir)
@@ -298,6 +300,7 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
            "int64": int(policy.get("ipt_f64", _choose_ipt(kp, 8)))}
     if not has_reducer:
         ipt = {k: int(policy.get("ipt_flat", 8)) for k in ipt}
+    xcd_run = int(policy.get("xcd_run", DEFAULT_XCD_RUN))
 
     # ---- Params ---------------------------------------------------------------------------
     params, fill = [], []
@@ -414,7 +417,10 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         "dtypes": list(dtypes),
         "row_aligned_index_inputs": sorted({s["selector_name"] + "_idx" for s in selector_register
                                             if s["selector"] == 1 and kp.vars[s["name"]].stage == 2}),
-        "policy": {"block": block, "ipt": {k: ipt[k] for k in dtypes}},
+        # value tensors read at index `row` for every row of a tile (served from the merge path): they
+        # must hold at least num_rows items
+        "row_indexed_value_inputs": sorted({src for _, src, _, _ in kp.row_sources}),
+        "policy": {"block": block, "ipt": {k: ipt[k] for k in dtypes}, "xcd_run": xcd_run},
         "widths": {"exchange": kp.xch_width, "reduce": kp.red_width, "aggregate": kp.agg_width,
                    "row": kp.row_width},
     })
@@ -423,15 +429,19 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
 
     ctype = {"float32": "float", "float64": "double", "int64": "long"}
     enum = {"float32": "FLEXSPMV_F32", "float64": "FLEXSPMV_F64", "int64": "FLEXSPMV_I64"}
-    cases_run, cases_ws = [], []
+    cases_run, cases_ws, cases_tiling = [], [], []
     for d in dtypes:
         disp = f"flex::Dispatch<Graph<{ctype[d]}>, {block}, {ipt[d]}, {'true' if has_reducer else 'false'}>"
         cases_run.append(
             f"    case {enum[d]}: {{ Graph<{ctype[d]}>::Params p; Graph<{ctype[d]}>::fill(p, a); return {disp}::run(p, a); }}\n")
         cases_ws.append(f"    case {enum[d]}: return {disp}::workspace_bytes(num_rows, ne);\n")
+        cases_tiling.append(f"    case {enum[d]}: return {disp}::tiling(num_rows, ne, out);\n")
 
     src = f"""// Generated by flexspmv_amd.codegen.merged_gen_gpu for sub-graph "{ir.name}" ({ir.content_hash()}).
 // Do not edit: regenerate from the six-list description instead.
+#ifndef FLEX_TUNE_XCD_RUN
+#define FLEX_TUNE_XCD_RUN {xcd_run}
+#endif
 #include "flex_dispatch.hpp"
 
 namespace {{
@@ -508,6 +518,13 @@ int flexspmv_last_kernel_ms(float* ms) {{ return flex::last_kernel_ms(ms); }}
 size_t flexspmv_workspace_bytes(int32_t dtype, int64_t num_rows, int64_t ne) {{
   switch (dtype) {{
 {''.join(cases_ws)}    default: return 0;
+  }}
+}}
+
+int flexspmv_tiling(int32_t dtype, int64_t num_rows, int64_t ne, int32_t out[6]) {{
+  flex::g_last_error[0] = 0;
+  switch (dtype) {{
+{''.join(cases_tiling)}    default: return flex::fail(FLEXSPMV_ERR_BAD_DTYPE, "Unsupported dtype for ValueT: this library was not generated for it");
   }}
 }}
 

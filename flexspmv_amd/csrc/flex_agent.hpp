@@ -101,19 +101,42 @@ __device__ __forceinline__ int2 merge_path_search_interp(int diag, const int* __
   return make_int2(min(lo, num_rows), diag - lo);
 }
 
-// One search per tile boundary: coords[t] is where tile t starts, coords[num_tiles] where the path ends.
-__global__ void __launch_bounds__(256)
-tile_search_kernel(int num_tiles, int tile_items, const int* __restrict__ row_end, int num_rows, int nnz,
-                   int2* __restrict__ coords) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t > num_tiles) return;
-  const long long d = (long long)t * tile_items;
+// How a launch cuts the merge path into tiles.  Tile boundary t lies on diagonal t * nominal; with
+// snap_slack > 0 an interior boundary is moved back to the start of the nearest row whose index is a
+// multiple of (snap_mask + 1) when that costs at most snap_slack merge items.  nominal + snap_slack is
+// the tile capacity, so a tile never outgrows its block.  A tile that starts on such a row starts
+// whole output lines (no row shared with the previous tile, no carry into it) - worth the smaller
+// tiles where rows are short (meshes, stencils); the host turns it off where they are not.
+struct Tiling {
+  int num_tiles;
+  int nominal;     // merge items between two diagonals
+  int snap_slack;  // 0: boundaries stay on their diagonals
+  int snap_mask;   // rows per output line - 1 (power of two - 1)
+};
+
+__device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end, int num_rows,
+                                              int nnz) {
+  const long long d = (long long)t * tl.nominal;
   const int diag = (int)min(d, (long long)num_rows + nnz);
 #ifdef FLEX_TUNE_BISECTION_ONLY  // tuning switch: the reference's plain bisection
-  coords[t] = merge_path_search(diag, row_end, num_rows, nnz);
+  int2 c = merge_path_search(diag, row_end, num_rows, nnz);
 #else
-  coords[t] = merge_path_search_interp(diag, row_end, num_rows, nnz);
+  int2 c = merge_path_search_interp(diag, row_end, num_rows, nnz);
 #endif
+  if (tl.snap_slack > 0 && t > 0 && t < tl.num_tiles) {
+    const int xs = c.x & ~tl.snap_mask;
+    const int ys = xs > 0 ? row_end[xs - 1] : 0;  // first non-zero of row xs
+    if ((c.x - xs) + (c.y - ys) <= tl.snap_slack) c = make_int2(xs, ys);
+  }
+  return c;
+}
+
+// One search per tile boundary: coords[t] is where tile t starts, coords[num_tiles] where the path ends.
+__global__ void __launch_bounds__(256)
+tile_search_kernel(const Tiling tl, const int* __restrict__ row_end, int num_rows, int nnz, int2* __restrict__ coords) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t > tl.num_tiles) return;
+  coords[t] = tile_boundary(t, tl, row_end, num_rows, nnz);
 }
 
 // Which tile a block works on.  Blocks are dealt to the 8 XCDs round-robin (block % 8), each XCD with
@@ -181,13 +204,17 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
   static_assert((IPT & (IPT - 1)) == 0 && IPT <= 32, "a thread's items must sit inside one bitmap word");
   static_assert(NWORDS <= WAVE, "one wavefront scans the bitmap words");
 
-  // s_xch holds the per-edge values of the tile; the merge path reuses it (after a barrier) as its
-  // output buffer s_out
+  // s_xch holds the per-edge values of the tile, s_out the rows the merge path finishes.  Where both
+  // fit a modest budget they are separate; otherwise s_out reuses s_xch after a barrier.
+#ifndef FLEX_TUNE_SEPARATE_OUT_BYTES
+#define FLEX_TUNE_SEPARATE_OUT_BYTES (20 * 1024)
+#endif
   constexpr int XCH_ELEMS = XCHN * TILE, OUT_ELEMS = REDN * OUT_STRIDE;
-  __shared__ V s_xch[XCH_ELEMS > OUT_ELEMS ? XCH_ELEMS : OUT_ELEMS];
-  V* const s_out = s_xch;
+  constexpr bool SEPARATE_OUT = (size_t)(XCH_ELEMS + OUT_ELEMS) * sizeof(V) <= (size_t)FLEX_TUNE_SEPARATE_OUT_BYTES;
+  constexpr int LDS_ELEMS = SEPARATE_OUT ? XCH_ELEMS + OUT_ELEMS : (XCH_ELEMS > OUT_ELEMS ? XCH_ELEMS : OUT_ELEMS);
+  __shared__ V s_xch[LDS_ELEMS];
+  V* const s_out = SEPARATE_OUT ? s_xch + XCH_ELEMS : s_xch;
   __shared__ unsigned s_bits[NWORDS];
-  __shared__ int s_word_prefix[NWORDS];
   __shared__ int s_vote[NW];
   __shared__ int s_wave_key[NW];
   __shared__ V s_wave_val[NW][REDN];
@@ -335,7 +362,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
         G::store_row(p, x0 + r, tot);
       } else {  // r == R: the row still open at the end of the tile becomes the tile's carry
         const int row = x0 + r;
-        carry_row[tile] = (row < num_rows) ? row : -1;
+        carry_row[tile] = (row < num_rows && len > 0) ? row : -1;
 #pragma unroll
         for (int c = 0; c < RED; ++c) carry_val[(size_t)tile * RED + c] = tot.v[c];
       }
@@ -354,25 +381,30 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
       atomicOr(&s_bits[pos >> 5], 1u << (pos & 31));
     }
     __syncthreads();
-    // exclusive prefix of the bitmap's per-word popcounts
-    if (wave == 0) {
-      int cnt[1] = {lane < NWORDS ? (int)__popc(s_bits[lane < NWORDS ? lane : 0]) : 0};
+    // Every wavefront scans the bitmap for itself (lane l takes word l): the number of row ends before
+    // each word, then each thread picks up its own word and that word's count from the lane that holds
+    // them.  No second barrier, no LDS round trip.
+    unsigned word;
+    int word_prefix;
+    {
+      const unsigned my_word = s_bits[lane < NWORDS ? lane : 0];
+      int cnt[1] = {lane < NWORDS ? (int)__popc(my_word) : 0};
       const int own = cnt[0];
       wave_segmented_inclusive_sum<int, 1>(0, cnt);
-      if (lane < NWORDS) s_word_prefix[lane] = cnt[0] - own;
+      const int src_lane = (tid * IPT) >> 5;  // < NWORDS <= WAVE
+      word = (unsigned)__builtin_amdgcn_ds_bpermute(src_lane << 2, (int)my_word);
+      word_prefix = __builtin_amdgcn_ds_bpermute(src_lane << 2, cnt[0] - own);
     }
-    __syncthreads();
 
     // this thread's IPT merge items
     const int tile_items = R + Z;
     const int d0 = tid * IPT;
     const int n_items = max(0, min(IPT, tile_items - d0));
-    const unsigned word = s_bits[d0 >> 5];
     const int sh = d0 & 31;
     constexpr unsigned FULL = (IPT == 32) ? 0xffffffffu : ((1u << IPT) - 1u);
     const unsigned ends = (word >> sh) & FULL;                                        // items that are row ends
     const unsigned nzs = ~ends & (n_items >= IPT ? FULL : ((1u << n_items) - 1u));  // ... that are non-zeros
-    const int xs = s_word_prefix[d0 >> 5] + __popc(word & ((1u << sh) - 1u));        // rows before my items
+    const int xs = word_prefix + __popc(word & ((1u << sh) - 1u));                    // rows before my items
     const int ys = d0 - xs;                                                            // non-zeros before them
 
     Pack<V, XCH> xv[IPT];
@@ -386,7 +418,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
       for (int c = 0; c < XCH; ++c) xv[it].v[c] = s_xch[c * TILE + yi];
     }
 
-    __syncthreads();  // every thread has read its s_xch values: the buffer now serves as s_out
+    if constexpr (!SEPARATE_OUT) __syncthreads();  // every thread has read its s_xch values: the buffer now serves as s_out
 
     Pack<V, RED> tot;
     zero(tot);
@@ -481,8 +513,11 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
 #pragma unroll
         for (int c = 0; c < RED; ++c) run[c] += pv[c];
       }
+      // the open row has non-zeros in this tile unless the tile's last merge item is a row end
+      const int last_item = tile_items - 1;
+      const bool open_empty = Z == 0 || (R > 0 && ((s_bits[last_item >> 5] >> (last_item & 31)) & 1u) != 0u);
       const int row = x0 + key;
-      carry_row[tile] = (row < num_rows) ? row : -1;
+      carry_row[tile] = (row < num_rows && !open_empty) ? row : -1;
 #pragma unroll
       for (int c = 0; c < RED; ++c) carry_val[(size_t)tile * RED + c] = run[c];
     }
@@ -507,14 +542,22 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
   }
 }
 
-// One block per tile by default.  With FLEX_TUNE_PERSISTENT (tuning switch) a launch has at most that many
-// blocks per CU; each walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... and reads the coordinates of its next
-// tile while it works on the current one.
+// One block per tile.  The tile's coordinates come from the table tile_search_kernel wrote (coords !=
+// NULL), or - small launches, where a kernel of its own for the search costs more than the search -
+// from the block itself: lanes 0 and 1 search the two diagonals that bound the tile (the reference does
+// the same when its grid is smaller than the device, cuda_template/reducer/merged_spmv_template.cuh:97-119,
+// merged_agent_spmv_template.cuh:412-435).  coords_out != NULL makes such a block leave its
+// coordinates in the table all the same (a debugging aid: the table can then be read back).
+// With FLEX_TUNE_PERSISTENT (tuning switch) a launch has at most that many blocks per CU; each walks
+// tiles blockIdx.x, blockIdx.x + gridDim.x, ... and reads the coordinates of its next tile while it
+// works on the current one.
 template <class G, int BLOCK, int IPT>
 __global__ void __launch_bounds__(BLOCK)
-reduce_kernel(const int2* __restrict__ coords, const int num_tiles, const int num_rows, const int* __restrict__ row_end,
+reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_rows, const int* __restrict__ row_end,
               const int nnz, const typename G::Params p, int* __restrict__ carry_row,
-              typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials) {
+              typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials,
+              int2* __restrict__ coords_out) {
+  const int num_tiles = tl.num_tiles;
 #ifdef FLEX_TUNE_PERSISTENT
   int tile = blockIdx.x;
   if (tile >= num_tiles) return;
@@ -537,8 +580,26 @@ reduce_kernel(const int2* __restrict__ coords, const int num_tiles, const int nu
 #else
   const int tile = tile_of_block(blockIdx.x, num_tiles);
   if (tile >= num_tiles) return;
-  reduce_tile<G, BLOCK, IPT>(tile, coords[tile], coords[tile + 1], num_rows, row_end, nnz, p, carry_row, carry_val,
-                             agg_partials);
+  int2 c0, c1;
+  if (coords != nullptr) {
+    c0 = coords[tile];
+    c1 = coords[tile + 1];
+  } else {
+    __shared__ int2 s_coord[2];
+    if (threadIdx.x < 2) s_coord[threadIdx.x] = tile_boundary(tile + (int)threadIdx.x, tl, row_end, num_rows, nnz);
+    __syncthreads();
+    c0 = s_coord[0];
+    c1 = s_coord[1];
+    c0.x = __builtin_amdgcn_readfirstlane(c0.x);
+    c0.y = __builtin_amdgcn_readfirstlane(c0.y);
+    c1.x = __builtin_amdgcn_readfirstlane(c1.x);
+    c1.y = __builtin_amdgcn_readfirstlane(c1.y);
+    if (coords_out != nullptr && threadIdx.x == 0) {
+      coords_out[tile] = c0;
+      if (tile == num_tiles - 1) coords_out[num_tiles] = c1;
+    }
+  }
+  reduce_tile<G, BLOCK, IPT>(tile, c0, c1, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
 #endif
 }
 
@@ -596,15 +657,18 @@ flat_kernel(const typename G::Params p, const int nnz, const int num_tiles,
 }
 
 // ----------------------------------------------------------------------------------------------
-// Fix-up: fold tile carries into their rows (tile order) and pre-reduce the aggregator partials.
-// Block b handles tiles [b*BLOCK, (b+1)*BLOCK): a thread owns the carry of one tile and, when it is
-// the first tile of a run that carries into the same row, adds the whole run to that row.  The
-// block's aggregator partials (PARTS_PER_TILE per tile, one per wavefront of the reducer block) are
-// summed in a fixed order into block_partials[b]; aggregate_kernel adds those, again in a fixed order.
+// Fix-up: fold tile carries into their rows (tile order) and reduce the aggregator partials.
+// A thread owns the carry of one tile at a time and, when that tile is the first of a run that carries
+// into the same row, adds the whole run to that row.  The aggregator partials (PARTS_PER_TILE per tile,
+// one per wavefront of the reducer block) are summed in a fixed order.
+//   SINGLE = false: block b handles tiles [b*BLOCK, (b+1)*BLOCK) and leaves its sum in block_partials[b];
+//                   aggregate_kernel adds those, again in a fixed order.
+//   SINGLE = true:  one block walks all tiles (launches of a few thousand tiles) and assigns the
+//                   aggregator outputs itself: one kernel less.
 // (Finishing the sum in the last fix-up block to finish, found with a ticket counter, was measured and
 // is slower: the release fence each block needs writes the XCD's whole L2 back, output rows included.)
 // ----------------------------------------------------------------------------------------------
-template <class G, int BLOCK, int PARTS_PER_TILE>
+template <class G, int BLOCK, int PARTS_PER_TILE, bool SINGLE>
 __global__ void __launch_bounds__(BLOCK)
 fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restrict__ carry_row,
              const typename G::Value* __restrict__ carry_val, const typename G::Value* __restrict__ agg_partials,
@@ -612,9 +676,12 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
   using V = typename G::Value;
   constexpr int RED = G::RED_WIDTH, AGG = G::AGG_WIDTH;
   constexpr int NW = BLOCK / WAVE;
-  const int t = blockIdx.x * BLOCK + threadIdx.x;
-  if constexpr (RED > 0) {
-    if (t < num_tiles) {
+  const int first = SINGLE ? (int)threadIdx.x : (int)(blockIdx.x * BLOCK + threadIdx.x);
+  const int stride = SINGLE ? BLOCK : num_tiles;  // not SINGLE: one tile per thread
+  Pack<V, AGG> acc;
+  zero(acc);
+  for (int t = first; t < num_tiles; t += stride) {
+    if constexpr (RED > 0) {
       const int row = carry_row[t];
       if (row >= 0 && !(t > 0 && carry_row[t - 1] == row)) {  // first tile of this row's run
         Pack<V, RED> sum;
@@ -627,18 +694,16 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
         G::add_row(p, row, sum);
       }
     }
-  }
-  if constexpr (AGG > 0) {
-    __shared__ V s_wave_agg[NW][AGG];
-    Pack<V, AGG> acc;
-    zero(acc);
-    if (t < num_tiles) {
+    if constexpr (AGG > 0) {
 #pragma unroll
       for (int w = 0; w < PARTS_PER_TILE; ++w) {
 #pragma unroll
         for (int c = 0; c < AGG; ++c) acc.v[c] += agg_partials[((size_t)t * PARTS_PER_TILE + w) * AGG + c];
       }
     }
+  }
+  if constexpr (AGG > 0) {
+    __shared__ V s_wave_agg[NW][AGG];
     wave_sum_to_last_lane<V, AGG>(acc.v);
     if ((threadIdx.x & (WAVE - 1)) == WAVE - 1) {
 #pragma unroll
@@ -646,11 +711,18 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
     }
     __syncthreads();
     if (threadIdx.x == 0) {
+      Pack<V, AGG> total;
 #pragma unroll
       for (int c = 0; c < AGG; ++c) {
         V s = s_wave_agg[0][c];
         for (int w = 1; w < NW; ++w) s += s_wave_agg[w][c];
-        block_partials[(size_t)blockIdx.x * AGG + c] = s;
+        total.v[c] = s;
+      }
+      if constexpr (SINGLE) {
+        G::store_agg(p, total);
+      } else {
+#pragma unroll
+        for (int c = 0; c < AGG; ++c) block_partials[(size_t)blockIdx.x * AGG + c] = total.v[c];
       }
     }
   }

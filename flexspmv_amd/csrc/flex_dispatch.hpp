@@ -74,23 +74,63 @@ inline int resident_grid(KernelT kernel, int block_threads, GridCache& cache) {
   return grid;
 }
 
+// Launch-shape policy (tuning switches in capitals; the defaults are what measured best on MI355X).
+#ifndef FLEX_TUNE_SNAP_BYTES
+#define FLEX_TUNE_SNAP_BYTES 128  // tiles start on rows whose outputs start a line of this many bytes (0: never)
+#endif
+#ifndef FLEX_TUNE_INBLOCK_MAX_TILES
+#define FLEX_TUNE_INBLOCK_MAX_TILES 8192  // launches of at most this many tiles search inside the reducer blocks
+#endif
+#ifndef FLEX_TUNE_SINGLE_FIXUP_MAX_TILES
+#define FLEX_TUNE_SINGLE_FIXUP_MAX_TILES 8192  // ... and fold carries and aggregators in one block
+#endif
+constexpr int SINGLE_FIXUP_BLOCK = 1024;
+
 template <class G, int BLOCK, int IPT, bool REDUCER>
 struct Dispatch {
   using V = typename G::Value;
   static constexpr int TILE = BLOCK * IPT;
 
   struct Layout {
+    Tiling tiling;
     int num_tiles;
     int flat_blocks;
     int carry_blocks;
+    bool search_in_blocks;
+    bool single_fixup;
     size_t off_coords, off_carry_row, off_carry_val, off_partials, off_block_partials, total;
   };
+
+  // Row-snapped tiles pay with smaller tiles (capacity minus the slack a boundary may be moved by), so
+  // they are used where a line's worth of rows is a small part of a tile: the slack is the merge items
+  // of that many average rows, and snapping is off when it exceeds an eighth of the tile.
+  static Tiling tiling_for(int64_t num_rows, int64_t ne) {
+    Tiling t;
+    t.nominal = TILE;
+    t.snap_slack = 0;
+    t.snap_mask = 0;
+    if (REDUCER && FLEX_TUNE_SNAP_BYTES > 0 && num_rows > 0) {
+      const int snap_rows = FLEX_TUNE_SNAP_BYTES / (int)sizeof(V) > 1 ? FLEX_TUNE_SNAP_BYTES / (int)sizeof(V) : 1;
+      const int64_t slack = (snap_rows * (num_rows + ne) + num_rows - 1) / num_rows;  // snap_rows average rows
+      if (slack <= TILE / 8) {
+        t.snap_slack = (int)slack;
+        t.snap_mask = snap_rows - 1;
+        t.nominal = TILE - (int)slack;
+      }
+    }
+    const int64_t items = REDUCER ? num_rows + ne : ne;
+    t.num_tiles = (int)((items + t.nominal - 1) / t.nominal);
+    return t;
+  }
 
   static bool layout(int64_t num_rows, int64_t ne, Layout& l) {
     const int64_t items = REDUCER ? num_rows + ne : ne;
     if (items <= 0 || num_rows + ne >= ((int64_t)1 << 31) - TILE) return false;
-    l.num_tiles = (int)((items + TILE - 1) / TILE);
+    l.tiling = tiling_for(num_rows, ne);
+    l.num_tiles = l.tiling.num_tiles;
     l.flat_blocks = l.num_tiles < MAX_PERSISTENT_BLOCKS ? l.num_tiles : MAX_PERSISTENT_BLOCKS;
+    l.search_in_blocks = REDUCER && l.num_tiles <= FLEX_TUNE_INBLOCK_MAX_TILES;
+    l.single_fixup = REDUCER && l.num_tiles <= FLEX_TUNE_SINGLE_FIXUP_MAX_TILES;
     size_t off = 0;
     l.off_coords = off;
     if (REDUCER) off += align_up(sizeof(int2) * ((size_t)l.num_tiles + 1));
@@ -114,22 +154,46 @@ struct Dispatch {
     return l.total;
   }
 
-  static int run(const typename G::Params& p, const flexspmv_launch_args* a) {
-    static thread_local GridCache grid_cache;  // one per kernel instantiation and host thread
+  static int tiling(int64_t num_rows, int64_t ne, int32_t* out) {
     Layout l;
+    if (out == nullptr) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "out is NULL");
+    if (!layout(num_rows, ne, l))
+      return fail(FLEXSPMV_ERR_TOO_LARGE, "num_rows + ne must be positive and stay below 2^31 (32-bit offsets)");
+    out[0] = l.tiling.num_tiles;
+    out[1] = l.tiling.nominal;
+    out[2] = l.tiling.snap_slack;
+    out[3] = l.tiling.snap_mask + 1;
+    out[4] = TILE;
+    out[5] = l.search_in_blocks ? 1 : 0;
+    return FLEXSPMV_OK;
+  }
+
+  // Checks shared by every entry point that launches: sizes, workspace, row pointer.
+  static int check(const flexspmv_launch_args* a, Layout& l, size_t workspace_bytes_available) {
     if (a->ne <= 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "selector index must be non-empty (ne > 0)");
     if (REDUCER && a->num_rows <= 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "num_rows must be positive");
     if (!layout(a->num_rows, a->ne, l))
       return fail(FLEXSPMV_ERR_TOO_LARGE, "num_rows + ne must stay below 2^31 (32-bit offsets)");
-    if (l.total > 0 && (a->workspace == nullptr || a->workspace_bytes < l.total))
+    if (l.total > workspace_bytes_available)
       return fail(FLEXSPMV_ERR_WORKSPACE, "workspace is missing or smaller than flexspmv_workspace_bytes()");
     if (REDUCER && a->row_end_offsets == nullptr)
       return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "row_end_offsets is required by a reducer sub-graph");
+    return FLEXSPMV_OK;
+  }
 
+  static int run(const typename G::Params& p, const flexspmv_launch_args* a) {
+    Layout l;
+    const int bad = check(a, l, a->workspace == nullptr ? 0 : a->workspace_bytes);
+    if (bad != FLEXSPMV_OK) return bad;
+    return launch(p, a, l, (char*)a->workspace);
+  }
+
+  // The kernels of one launch, on a->stream, with scratch at ws (l.total bytes, 256-byte aligned).
+  static int launch(const typename G::Params& p, const flexspmv_launch_args* a, const Layout& l, char* ws) {
+    static thread_local GridCache grid_cache;  // one per kernel instantiation and host thread
     hipStream_t stream = (hipStream_t)a->stream;
     const bool timed = (a->flags & FLEXSPMV_FLAG_TIME_KERNEL) != 0 && g_timer.ready();
     g_timer.armed = false;
-    char* ws = (char*)a->workspace;
     V* partials = (V*)(ws + l.off_partials);
     const int nnz = (int)a->ne;
 
@@ -140,10 +204,10 @@ struct Dispatch {
       int* carry_row = (int*)(ws + l.off_carry_row);
       V* carry_val = (V*)(ws + l.off_carry_val);
 
-      if ((a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0) {
+      if (!l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0) {
         const int search_blocks = (l.num_tiles + 1 + 255) / 256;
-        hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(256), 0, stream, l.num_tiles, TILE,
-                           row_end, num_rows, nnz, coords);
+        hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(256), 0, stream, l.tiling, row_end, num_rows,
+                           nnz, coords);
       }
       if (timed) (void)hipEventRecord(g_timer.start, stream);
 #ifdef FLEX_TUNE_PERSISTENT
@@ -151,15 +215,24 @@ struct Dispatch {
 #else
       const int reduce_grid = grid_for_tiles(l.num_tiles);
 #endif
-      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(reduce_grid), dim3(BLOCK), 0, stream,
-                         (const int2*)coords, l.num_tiles, num_rows, row_end, nnz, p, carry_row, carry_val, partials);
+      const int2* table = l.search_in_blocks ? nullptr : coords;
+      int2* table_out = (l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_KEEP_TILES) != 0) ? coords : nullptr;
+      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(reduce_grid), dim3(BLOCK), 0, stream, table, l.tiling,
+                         num_rows, row_end, nnz, p, carry_row, carry_val, partials, table_out);
       if (timed) g_timer.armed = (hipEventRecord(g_timer.stop, stream) == hipSuccess);
       V* block_partials = (V*)(ws + l.off_block_partials);
-      hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, BLOCK / WAVE>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0, stream, p,
-                         l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials, block_partials);
-      if (G::AGG_WIDTH > 0) {
-        hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
-                           (const V*)block_partials, l.carry_blocks);
+      if (l.single_fixup) {
+        hipLaunchKernelGGL((fixup_kernel<G, SINGLE_FIXUP_BLOCK, BLOCK / WAVE, true>), dim3(1), dim3(SINGLE_FIXUP_BLOCK), 0,
+                           stream, p, l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials,
+                           block_partials);
+      } else {
+        hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, BLOCK / WAVE, false>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0,
+                           stream, p, l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials,
+                           block_partials);
+        if (G::AGG_WIDTH > 0) {
+          hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
+                             (const V*)block_partials, l.carry_blocks);
+        }
       }
     } else {
       int grid = resident_grid(flat_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
@@ -183,7 +256,7 @@ inline int check_counts(const flexspmv_launch_args* a, int nv, int ni, int no) {
   if (a == nullptr) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "args is NULL");
   if (a->struct_size != sizeof(flexspmv_launch_args))
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "struct_size does not match this library's flexspmv_launch_args");
-  if ((a->flags & ~(FLEXSPMV_FLAG_TIME_KERNEL | FLEXSPMV_FLAG_REUSE_TILES)) != 0)
+  if ((a->flags & ~(FLEXSPMV_FLAG_TIME_KERNEL | FLEXSPMV_FLAG_REUSE_TILES | FLEXSPMV_FLAG_KEEP_TILES)) != 0)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "unknown bits in flags");
   if (a->num_value_inputs != nv || a->num_index_inputs != ni || a->num_outputs != no)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "argument counts do not match flexspmv_signature()");

@@ -32,7 +32,9 @@ def capture_step(compiled, warmup: int = 2) -> Callable[[], None]:
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    # captured on the stream the warm-up ran on: every library keeps one scratch buffer per stream and
+    # must not allocate a new one inside the capture
+    with torch.cuda.graph(graph, stream=side):
         compiled()
     # the capture itself does not execute: the model is where the warm-up left it
 

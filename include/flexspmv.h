@@ -1,7 +1,7 @@
 /* C interface of a generated FlexSpmv library for MI355X (gfx950).
  *
  * One shared library is generated per fused sub-graph (select -> map -> reduce / aggregate).  Every
- * such library exports the same six symbols below; nothing in the signatures is a torch type, so
+ * such library exports the same symbols below; nothing in the signatures is a torch type, so
  * any host (Python ctypes, a torch extension, C++) can bind them.
  *
  * What each entry point stands in for in the reference:
@@ -17,6 +17,9 @@
  *                             (codegen/merged_gen_binding.py:27-78,112-134); here it is data.
  *   flexspmv_last_error       the strings TORCH_CHECK raises (cuda_template/merged_binding_template.cu:40-50).
  *   flexspmv_abi_version      no counterpart; lets a loader reject a stale library.
+ *   flexspmv_tiling           the tile arithmetic of the reference's dispatch (num_merge_tiles from
+ *                             num_rows + num_nonzeros and the policy's tile size,
+ *                             cuda_template/reducer/merged_spmv_template.cuh:60-80), as data.
  *   flexspmv_last_kernel_ms   the GpuTimer bracket of the reference's CUDA harness
  *                             (src/flex_spmv_full_red.cu:298-330, utils.h:634-669), narrowed to the
  *                             dominant kernel of one launch so that a roofline can be measured live.
@@ -31,7 +34,7 @@
 extern "C" {
 #endif
 
-#define FLEXSPMV_ABI_VERSION 2
+#define FLEXSPMV_ABI_VERSION 3
 
 /* flexspmv_launch_args.flags */
 #define FLEXSPMV_FLAG_TIME_KERNEL 1u /* bracket the dominant kernel with HIP events on args->stream */
@@ -41,6 +44,11 @@ extern "C" {
  * is then reused (the reference recomputes it on every call, include/merged_spmv_kernels.cuh:60-99;
  * a solver iterating on a fixed sparsity pattern needs it once). */
 #define FLEXSPMV_FLAG_REUSE_TILES 2u
+/* Leave the tile table (int32 pairs (rows, non-zeros) for tile boundaries 0 .. num_tiles, at the start
+ * of the workspace) behind even when the launch is small enough for the reducer blocks to search their
+ * own boundaries and would not write it.  A debugging aid: the table of any launch can be read back
+ * and compared with a CPU merge-path search (see flexspmv_tiling for the diagonals). */
+#define FLEXSPMV_FLAG_KEEP_TILES 4u
 
 /* Value types a library may have been generated for (flexspmv_launch_args.dtype). */
 enum flexspmv_dtype { FLEXSPMV_F32 = 0, FLEXSPMV_F64 = 1, FLEXSPMV_I64 = 2 };
@@ -59,7 +67,10 @@ enum flexspmv_status {
  *                  sources (order of first use); row-major [n][Dim], contiguous.  In-place map ops
  *                  (setitem / copy_ / add_) write through these pointers.
  *   index_inputs   one int32 array of ne entries per unique selector module, binding order.  An array
- *                  declared row-aligned in flexspmv_signature() is never dereferenced.
+ *                  listed under "row_aligned_index_inputs" in flexspmv_signature() is never dereferenced:
+ *                  the caller guarantees that it equals the row id of every edge, and the value inputs
+ *                  listed under "row_indexed_value_inputs" are then read at every row id 0 .. num_rows-1
+ *                  (rows without edges included), so they must hold at least num_rows items.
  *   outputs        one buffer per output in binding order: reducer [num_rows][Dim], aggregator [Dim],
  *                  map output [ne][Dim].  Every element is overwritten; no zero fill is needed.
  *   row_end_offsets  int32[num_rows + 1] with a leading 0 (CSR row pointer); ignored (may be NULL) by
@@ -107,6 +118,19 @@ const char* flexspmv_last_error(void);
  * FLEXSPMV_FLAG_TIME_KERNEL.  Blocks until that kernel has finished.  Returns FLEXSPMV_OK, or
  * FLEXSPMV_ERR_BAD_ARGUMENT when no such launch was made. */
 int flexspmv_last_kernel_ms(float* ms);
+
+/* How a launch of these sizes cuts the merge path of (row end offsets, 0 .. ne-1) into tiles:
+ *   out[0] num_tiles     tile t covers the path from boundary t to boundary t + 1
+ *   out[1] nominal       boundary t lies on diagonal min(t * nominal, num_rows + ne) ...
+ *   out[2] snap_slack    ... unless 0 < t < num_tiles and the start of row (x & ~(snap_rows - 1)), x the
+ *   out[3] snap_rows     row coordinate on that diagonal, is at most snap_slack merge items back: then the
+ *                        boundary is that row start.  snap_slack = 0: boundaries stay on their diagonals.
+ *   out[4] tile_capacity merge items a block can hold (nominal + snap_slack)
+ *   out[5] search_in_blocks  1 when the reducer blocks search their own boundaries (no table is written
+ *                        unless FLEXSPMV_FLAG_KEEP_TILES is given), else 0
+ * For libraries without a reducer the tiles are plain edge ranges of `nominal` edges.
+ * Returns FLEXSPMV_OK, FLEXSPMV_ERR_BAD_DTYPE or FLEXSPMV_ERR_TOO_LARGE. */
+int flexspmv_tiling(int32_t dtype, int64_t num_rows, int64_t ne, int32_t out[6]);
 
 /* FLEXSPMV_ABI_VERSION the library was built against. */
 int flexspmv_abi_version(void);

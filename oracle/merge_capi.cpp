@@ -12,6 +12,16 @@ void oracle_merge_path_search(int diagonal, const int* row_end, int num_rows, in
   out_xy[1] = c.y;
 }
 
+// the same for n diagonals: out_xy[2*i], out_xy[2*i+1] for diagonals[i]
+void oracle_merge_path_search_many(const int* diagonals, int n, const int* row_end, int num_rows, int nnz, int* out_xy) {
+  oracle::Counting nz(0);
+  for (int i = 0; i < n; ++i) {
+    const oracle::Coord c = oracle::merge_path_search(diagonals[i], row_end, nz, num_rows, nnz);
+    out_xy[2 * i] = c.x;
+    out_xy[2 * i + 1] = c.y;
+  }
+}
+
 // begin/end coordinates of thread tid: out = {begin.x, begin.y, end.x, end.y}
 void oracle_reducer_thread_span(int tid, int num_threads, const int* row_end, int num_rows, int nnz, int* out) {
   const oracle::Span s = oracle::reducer_thread_span(tid, num_threads, row_end, num_rows, nnz);

@@ -1,0 +1,136 @@
+"""The tile table the device computes, bit for bit against the CPU merge-path search.
+
+Reference: MergePathSearch (include/merged_spmv_kernels.cuh:19-50, CPU twin
+cpu_template/merged_spmv_template_reducer.h:27-51) as driven by SpmvSearchKernel (:60-99): one search per
+tile boundary on diagonal t * tile_items.  The device search (flex_agent.hpp: a few interpolation probes,
+then bisection - in tile_search_kernel, or inside the reducer blocks for small launches) must give exactly
+the coordinates of the reference's plain bisection, restated in oracle/merge_ref.hpp and pinned there
+against the reference's own code.  Where the launch moves a boundary back to a row start (row-snapped
+tiles, a rule of this library stated in include/flexspmv.h), the expected coordinate is that row start and
+the condition is evaluated from the oracle's coordinate.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+from flexspmv_amd import graphs
+from flexspmv_amd import workloads as W
+from flexspmv_amd.binding import DTYPE_CODES, FLAG_KEEP_TILES, load_named
+from oracle import build_oracle
+from tests.test_gpu_parity import case_rng
+from tests.util_inputs import STRUCTURES, make_inputs, random_row_structure, row_structure
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def merge_lib():
+    lib = ctypes.CDLL(build_oracle.build_merge_capi())
+    lib.oracle_merge_path_search_many.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+                                                  ctypes.c_int, ctypes.c_void_p]
+    return lib
+
+
+def tiling_of(ext, dtype, num_rows, ne):
+    out = (ctypes.c_int32 * 6)()
+    rc = ext._lib.flexspmv_tiling(DTYPE_CODES[dtype], num_rows, ne, out)
+    assert rc == 0, ext._lib.flexspmv_last_error().decode()
+    return dict(zip(("num_tiles", "nominal", "snap_slack", "snap_rows", "capacity", "search_in_blocks"), out))
+
+
+def expected_table(merge_lib, row_ptr, tl):
+    """Tile boundaries 0 .. num_tiles from the oracle's search plus the snapping rule."""
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+    row_end = np.ascontiguousarray(row_ptr[1:])
+    num_rows, nnz = len(row_end), int(row_ptr[-1])
+    t = np.arange(tl["num_tiles"] + 1, dtype=np.int64)
+    diag = np.minimum(t * tl["nominal"], num_rows + nnz).astype(np.int32)
+    xy = np.empty((len(t), 2), dtype=np.int32)
+    merge_lib.oracle_merge_path_search_many(diag.ctypes.data, len(t), row_end.ctypes.data, num_rows, nnz,
+                                            xy.ctypes.data)
+    assert np.array_equal(xy.sum(axis=1), diag)                      # a point on its diagonal
+    if tl["snap_slack"] > 0:
+        x, y = xy[:, 0].astype(np.int64), xy[:, 1].astype(np.int64)
+        xs = x & ~np.int64(tl["snap_rows"] - 1)
+        ys = row_ptr[xs].astype(np.int64)                            # first non-zero of row xs
+        interior = (t > 0) & (t < tl["num_tiles"])
+        snap = interior & ((x - xs) + (y - ys) <= tl["snap_slack"])
+        xy[snap, 0] = xs[snap]
+        xy[snap, 1] = ys[snap]
+    return xy
+
+
+def device_table(name, dtype, tensors, row_ptr, num_rows, num_cols):
+    """Launch the library with FLEXSPMV_FLAG_KEEP_TILES and read the table back from its workspace."""
+    ext = load_named(name, build_if_missing=False)
+    args = []
+    for pname in ext.param_names():
+        if pname == "row_end_offsets":
+            args.append(torch.from_numpy(np.ascontiguousarray(row_ptr)).cuda())
+        elif pname in ("num_rows", "num_cols"):
+            args.append(int(num_rows if pname == "num_rows" else num_cols))
+        else:
+            t = tensors[pname]
+            args.append(t if isinstance(t, torch.Tensor) else torch.from_numpy(np.ascontiguousarray(t)).cuda())
+    ext.extra_flags = FLAG_KEEP_TILES
+    try:
+        ext.merged_spmv_launch(*args)
+    finally:
+        ext.extra_flags = 0
+    torch.cuda.synchronize()
+    ne = int(row_ptr[-1])
+    tl = tiling_of(ext, dtype, num_rows, ne)
+    ws = ext.workspace_of(torch.device("cuda", torch.cuda.current_device()))
+    table = ws[: 8 * (tl["num_tiles"] + 1)].view(torch.int32).view(-1, 2).cpu().numpy()
+    return table, tl
+
+
+def check_table(merge_lib, name, dtype, tensors, row_ptr, num_rows, num_cols):
+    table, tl = device_table(name, dtype, tensors, row_ptr, num_rows, num_cols)
+    want = expected_table(merge_lib, row_ptr, tl)
+    assert table.shape == want.shape
+    bad = np.nonzero((table != want).any(axis=1))[0]
+    assert bad.size == 0, (f"{name}: {bad.size} of {len(want)} tile boundaries differ, first at tile {bad[0]}: "
+                           f"device {table[bad[0]]} oracle {want[bad[0]]} ({tl})")
+    sizes = np.diff(table.sum(axis=1))
+    assert sizes.min() >= 0 and sizes.max() <= tl["capacity"]        # every tile fits its block
+    assert tuple(table[0]) == (0, 0) and tuple(table[-1]) == (num_rows, int(row_ptr[-1]))
+    return tl
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+@pytest.mark.parametrize("structure", STRUCTURES)
+def test_tile_table_on_every_row_structure(merge_lib, structure, dtype):
+    rng = case_rng("tile_table", structure)
+    row_ptr = row_structure(structure, rng)
+    for name in ("csr_spmv", "swe_rusanov"):                         # tiles of 2048 and of 1024 / 512 merge items
+        tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get(name), np.dtype(dtype), rng, row_ptr=row_ptr)
+        print(f"case tile table {name} {structure} {dtype} rows={nr} ne={ne}", flush=True)
+        check_table(merge_lib, name, dtype, tensors, row_ptr, nr, nc)
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_tile_table_on_random_row_structures(merge_lib, seed):
+    rng = np.random.default_rng(seed)
+    snapped = 0
+    for case in range(30):
+        dtype = ["float32", "float64"][int(rng.integers(0, 2))]
+        row_ptr = random_row_structure(rng)
+        tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get("csr_spmv"), np.dtype(dtype), rng, row_ptr=row_ptr)
+        print(f"case tile table random seed={seed} #{case} {dtype} rows={nr} ne={ne}", flush=True)
+        tl = check_table(merge_lib, "csr_spmv", dtype, tensors, row_ptr, nr, nc)
+        snapped += tl["snap_slack"] > 0
+    assert 0 < snapped < 30          # both kinds of tiling were exercised
+
+
+def test_tile_table_of_the_two_large_workloads(merge_lib):
+    """Poisson 256^3 (65 k+ tiles, written by tile_search_kernel, row-snapped) and R-MAT scale 22 (35 k tiles,
+    boundaries on their diagonals)."""
+    for w, dtype in ((W.poisson_3d_spmv_dot(256), "float64"), (W.rmat_spmv(22), "float32")):
+        print(f"case tile table {w.name} rows={w.num_rows} ne={w.ne}", flush=True)
+        tl = check_table(merge_lib, w.graph, dtype, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols)
+        assert tl["search_in_blocks"] == 0
+        print(f"  {tl}", flush=True)

@@ -155,7 +155,7 @@ def test_launch_rejects_bad_arguments_without_touching_the_gpu():
     err = lambda: lib.flexspmv_last_error().decode()
     assert lib.flexspmv_launch(None) == -1
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, struct_size=8))) == -1 and "struct_size" in err()
-    assert lib.flexspmv_launch(ctypes.byref(_args(lib, flags=6))) == -1
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, flags=8))) == -1 and "flags" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, num_value_inputs=1))) == -1 and "counts" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, dtype=2))) == -2 and "Unsupported dtype" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, ne=0))) == -1 and "non-empty" in err()
@@ -164,6 +164,24 @@ def test_launch_rejects_bad_arguments_without_touching_the_gpu():
     assert lib.flexspmv_launch(ctypes.byref(_args(lib))) == -4 and "workspace" in err()       # no scratch given
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, workspace=0x1000, workspace_bytes=1 << 20,
                                                   row_end_offsets=0))) == -1 and "row_end_offsets" in err()
+
+
+def test_tiling_query():
+    """flexspmv_tiling: tile count, diagonal spacing and the row-snapping parameters of a launch."""
+    lib = _lib("spmv_dot")
+    out = (ctypes.c_int32 * 6)()
+    # Poisson 256^3 in float64: 8 merge items per row, 16 rows per 128-byte output line -> slack 128
+    assert lib.flexspmv_tiling(1, 16777216, 117047296, out) == 0
+    num_tiles, nominal, slack, snap_rows, capacity, in_blocks = list(out)
+    assert (nominal, slack, snap_rows, capacity, in_blocks) == (2048 - 128, 128, 16, 2048, 0)
+    assert num_tiles == -(-(16777216 + 117047296) // nominal)
+    # long rows: a line's worth of rows is more than an eighth of a tile -> boundaries stay on their diagonals
+    assert lib.flexspmv_tiling(1, 1000, 1000 * 300, out) == 0
+    assert list(out)[1:5] == [2048, 0, 1, 2048] and out[5] == 1
+    assert lib.flexspmv_tiling(2, 1000, 7000, out) == -2             # int64 not compiled into this library
+    assert lib.flexspmv_tiling(1, 2**30, 2**30, out) == -3
+    flat = _lib("mass_sum")
+    assert flat.flexspmv_tiling(0, 5, 100000, out) == 0 and list(out)[1:4] == [2048, 0, 1]
 
 
 def test_workspace_query():
