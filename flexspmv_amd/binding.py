@@ -28,13 +28,14 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 from . import build as _build
 from .ir import FusedGraphIR
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 FLAG_TIME_KERNEL = 1
 FLAG_REUSE_TILES = 2
 FLAG_KEEP_TILES = 4
 DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
 EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
-                    "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms", "flexspmv_tiling")
+                    "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms", "flexspmv_tiling",
+                    "flexspmv_launch_static")
 
 
 class LaunchArgs(ctypes.Structure):
@@ -73,6 +74,8 @@ def load_library(path: str) -> ctypes.CDLL:
     lib = ctypes.CDLL(path, mode=ctypes.RTLD_LOCAL)
     lib.flexspmv_launch.argtypes = [ctypes.POINTER(LaunchArgs)]
     lib.flexspmv_launch.restype = ctypes.c_int
+    lib.flexspmv_launch_static.argtypes = [ctypes.POINTER(LaunchArgs)]
+    lib.flexspmv_launch_static.restype = ctypes.c_int
     lib.flexspmv_workspace_bytes.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.c_int64]
     lib.flexspmv_workspace_bytes.restype = ctypes.c_size_t
     lib.flexspmv_signature.argtypes = []

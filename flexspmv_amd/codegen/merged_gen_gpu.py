@@ -429,11 +429,13 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
 
     ctype = {"float32": "float", "float64": "double", "int64": "long"}
     enum = {"float32": "FLEXSPMV_F32", "float64": "FLEXSPMV_F64", "int64": "FLEXSPMV_I64"}
-    cases_run, cases_ws, cases_tiling = [], [], []
+    cases_run, cases_ws, cases_tiling, cases_static = [], [], [], []
     for d in dtypes:
         disp = f"flex::Dispatch<Graph<{ctype[d]}>, {block}, {ipt[d]}, {'true' if has_reducer else 'false'}>"
         cases_run.append(
             f"    case {enum[d]}: {{ Graph<{ctype[d]}>::Params p; Graph<{ctype[d]}>::fill(p, a); return {disp}::run(p, a); }}\n")
+        cases_static.append(
+            f"    case {enum[d]}: {{ Graph<{ctype[d]}>::Params p; Graph<{ctype[d]}>::fill(p, a); return {disp}::run_static(p, a); }}\n")
         cases_ws.append(f"    case {enum[d]}: return {disp}::workspace_bytes(num_rows, ne);\n")
         cases_tiling.append(f"    case {enum[d]}: return {disp}::tiling(num_rows, ne, out);\n")
 
@@ -534,6 +536,15 @@ int flexspmv_launch(const flexspmv_launch_args* a) {{
   if (bad != FLEXSPMV_OK) return bad;
   switch (a->dtype) {{
 {''.join(cases_run)}    default: return flex::fail(FLEXSPMV_ERR_BAD_DTYPE, "Unsupported dtype for ValueT: this library was not generated for it");
+  }}
+}}
+
+int flexspmv_launch_static(const flexspmv_launch_args* a) {{
+  flex::g_last_error[0] = 0;
+  const int bad = flex::check_counts(a, {len(plan.value_inputs)}, {len(plan.selector_inputs)}, {len(plan.outputs)});
+  if (bad != FLEXSPMV_OK) return bad;
+  switch (a->dtype) {{
+{''.join(cases_static)}    default: return flex::fail(FLEXSPMV_ERR_BAD_DTYPE, "Unsupported dtype for ValueT: this library was not generated for it");
   }}
 }}
 

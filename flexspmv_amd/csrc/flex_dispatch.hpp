@@ -11,8 +11,16 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "flex_agent.hpp"
 #include "flexspmv.h"
+
+// Scratch of flexspmv_launch_static: device memory that belongs to the library itself, so that entry point
+// never allocates.  One copy exists on every GPU the library is loaded on, at its own address; host code
+// reaches it only through the per-device pointer that static_scratch() resolves (the array's name is
+// a host-side stand-in, not a device address).
+static __device__ __align__(256) unsigned char scratch[FLEXSPMV_STATIC_SCRATCH_BYTES];
 
 namespace flex {
 
@@ -42,6 +50,35 @@ inline int last_kernel_ms(float* ms) {
   if (e == hipSuccess) e = hipEventElapsedTime(ms, g_timer.start, g_timer.stop);
   if (e != hipSuccess) return fail_hip(e, "reading kernel timer");
   return FLEXSPMV_OK;
+}
+
+// Address of `scratch` on the current device, resolved once per device (the first call on a device asks
+// the runtime; later calls read the table).  NULL with g_last_error set when the runtime refuses.
+constexpr int MAX_DEVICES = 64;
+inline char* static_scratch() {
+  static std::mutex lock;
+  static void* table[MAX_DEVICES] = {};
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) {
+    fail_hip(e, "hipGetDevice");
+    return nullptr;
+  }
+  if (device < 0 || device >= MAX_DEVICES) {
+    fail(FLEXSPMV_ERR_BAD_ARGUMENT, "device ordinal beyond the static scratch table");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(lock);
+  if (table[device] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      fail_hip(e, "hipGetSymbolAddress(scratch)");
+      return nullptr;
+    }
+    table[device] = ptr;
+  }
+  return (char*)table[device];
 }
 
 constexpr size_t align_up(size_t n, size_t a = 256) { return (n + a - 1) / a * a; }
@@ -187,6 +224,26 @@ struct Dispatch {
     if (bad != FLEXSPMV_OK) return bad;
     return launch(p, a, l, (char*)a->workspace);
   }
+
+  // flexspmv_launch_static: the same launch with the library's own scratch; allocates nothing.
+  static int run_static(const typename G::Params& p, const flexspmv_launch_args* a) {
+    if ((a->flags & FLEXSPMV_FLAG_TIME_KERNEL) != 0)
+      return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "FLEXSPMV_FLAG_TIME_KERNEL creates events; flexspmv_launch_static does not take it");
+    Layout l;
+    const int bad = check(a, l, l_unbounded());
+    if (bad != FLEXSPMV_OK) return bad;
+    if (l.total > (size_t)FLEXSPMV_STATIC_SCRATCH_BYTES) {
+      snprintf(g_last_error, sizeof(g_last_error),
+               "flexspmv_launch_static: these sizes need %zu bytes of scratch, the library's static buffer holds %zu "
+               "(FLEXSPMV_STATIC_SCRATCH_BYTES); use flexspmv_launch with a caller-owned workspace",
+               l.total, (size_t)FLEXSPMV_STATIC_SCRATCH_BYTES);
+      return FLEXSPMV_ERR_WORKSPACE;
+    }
+    char* ws = static_scratch();
+    if (ws == nullptr) return FLEXSPMV_ERR_WORKSPACE;
+    return launch(p, a, l, ws);
+  }
+  static constexpr size_t l_unbounded() { return ~(size_t)0; }
 
   // The kernels of one launch, on a->stream, with scratch at ws (l.total bytes, 256-byte aligned).
   static int launch(const typename G::Params& p, const flexspmv_launch_args* a, const Layout& l, char* ws) {

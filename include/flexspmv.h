@@ -34,7 +34,10 @@
 extern "C" {
 #endif
 
-#define FLEXSPMV_ABI_VERSION 3
+#define FLEXSPMV_ABI_VERSION 4
+
+/* Scratch a library keeps for flexspmv_launch_static (bytes, per library and per GPU it is used on). */
+#define FLEXSPMV_STATIC_SCRATCH_BYTES (4u << 20)
 
 /* flexspmv_launch_args.flags */
 #define FLEXSPMV_FLAG_TIME_KERNEL 1u /* bracket the dominant kernel with HIP events on args->stream */
@@ -102,6 +105,20 @@ typedef struct flexspmv_launch_args {
 
 /* Run the fused sub-graph once.  Returns FLEXSPMV_OK, a negative flexspmv_status, or a hipError_t. */
 int flexspmv_launch(const flexspmv_launch_args* args);
+
+/* flexspmv_launch without any allocation.  No counterpart in the reference; it is for callers that cannot
+ * allocate device memory: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same arguments and results as flexspmv_launch, except that args->workspace / workspace_bytes are ignored:
+ * tile table, carries and aggregator partials live in a buffer of FLEXSPMV_STATIC_SCRATCH_BYTES that is part
+ * of the library's device image (one copy per GPU, held until the process ends).  The call makes no
+ * hipMalloc / hipFree and creates no events, so FLEXSPMV_FLAG_TIME_KERNEL is refused (BAD_ARGUMENT).  Sizes
+ * whose flexspmv_workspace_bytes() exceeds the buffer are refused with FLEXSPMV_ERR_WORKSPACE and a message
+ * that names both figures.  The first call on each GPU looks the buffer's address up (make it outside a
+ * capture); nothing in the buffer has to be cleared between calls - every word a launch reads it has
+ * written first.  All calls of one library on one GPU share the buffer: calls that overlap in time
+ * (two streams, two threads) race on it, and FLEXSPMV_FLAG_REUSE_TILES refers to the previous call of
+ * either entry point that used this buffer. */
+int flexspmv_launch_static(const flexspmv_launch_args* args);
 
 /* Scratch bytes flexspmv_launch needs for these sizes (0 is a valid answer). */
 size_t flexspmv_workspace_bytes(int32_t dtype, int64_t num_rows, int64_t ne);
