@@ -23,6 +23,7 @@ from __future__ import annotations
 import ctypes
 import json
 import os
+import threading
 from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 from . import build as _build
@@ -94,6 +95,21 @@ def load_library(path: str) -> ctypes.CDLL:
     return lib
 
 
+class _CallState:
+    """ctypes objects of one thread's launches of one library (kept alive together)."""
+    __slots__ = ("v_arr", "i_arr", "o_arr", "la", "ref")
+
+
+_DTYPE_NAMES: Dict[Any, str] = {}
+
+
+def _TORCH_DTYPE_NAMES() -> Dict[Any, str]:
+    if not _DTYPE_NAMES:
+        import torch
+        _DTYPE_NAMES.update({torch.float32: "float32", torch.float64: "float64", torch.int64: "int64"})
+    return _DTYPE_NAMES
+
+
 def _check(cond: bool, msg: str) -> None:
     if not cond:
         raise RuntimeError(msg)
@@ -131,6 +147,13 @@ class HipExtension:
         self.reuse_tiles = False
         self._tile_key = None
         self.extra_flags = 0       # FLAG_* bits added to every launch (FLAG_KEEP_TILES for debugging)
+        # what a launch looks up, prepared once
+        self._dispatch_name = self.signature["dispatch_tensor"]
+        self._tensor_names = self._value_names + self._index_names + ["row_end_offsets"]
+        self._dims = dict(self.signature["value_dims"])
+        self._out_specs = [(o["kind"], int(o["dim"])) for o in self._outputs]
+        self._ws_bytes: Dict[Any, int] = {}
+        self._tls = threading.local()
 
     # -- helpers -------------------------------------------------------------------------
     def param_names(self) -> List[str]:
@@ -151,8 +174,9 @@ class HipExtension:
     def workspace_bytes(self, dtype: str, num_rows: int, ne: int) -> int:
         return int(self._lib.flexspmv_workspace_bytes(DTYPE_CODES[dtype], num_rows, ne))
 
-    def _scratch(self, device, stream, nbytes: int):
-        """Scratch of this library for launches on ``stream`` of ``device``.
+    def _scratch(self, device, index: int, raw_stream: int, nbytes: int):
+        """Scratch of this library for launches on the stream with handle ``raw_stream`` of device ``index``
+        (the current stream of the current device when this is called).
 
         The buffer is allocated on that stream and only ever used on it, so when a larger launch replaces
         it the caching allocator hands the old block out again in stream order - nothing still running
@@ -160,17 +184,16 @@ class HipExtension:
         library (a replayed graph keeps using its address), and growing during a capture is refused:
         run the step once eagerly first, as capture_step does."""
         import torch
-        key = (device.index if device.index is not None else torch.cuda.current_device(), int(stream.cuda_stream))
-        capturing = torch.cuda.is_current_stream_capturing()
+        key = (index, raw_stream)
         buf = self._workspace.get(key)
+        capturing = torch._C._cuda_isCurrentStreamCapturing()
         if buf is None or buf.numel() < nbytes:
             _check(not capturing, "FlexSpmv scratch cannot grow during a stream capture: "
                                   "launch once with these sizes before capturing")
             if buf is not None and key in self._captured:
                 self._retained.append(buf)
                 self._captured.discard(key)
-            with torch.cuda.stream(stream):
-                buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+            buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
             self._workspace[key] = buf
         if capturing:
             self._captured.add(key)
@@ -186,100 +209,136 @@ class HipExtension:
         return self._workspace.get((index, int(stream.cuda_stream)))
 
     # -- the call ------------------------------------------------------------------------
+    def _call_state(self):
+        """Per-thread argument block of the C call, built once: the launch struct with its constant fields
+        and the three pointer arrays (a launch only rewrites pointers and sizes)."""
+        st = getattr(self._tls, "state", None)
+        if st is None:
+            nv, ni, no = len(self._value_names), len(self._index_names), len(self._outputs)
+            st = _CallState()
+            st.v_arr = (ctypes.c_void_p * max(nv, 1))()
+            st.i_arr = (ctypes.c_void_p * max(ni, 1))()
+            st.o_arr = (ctypes.c_void_p * max(no, 1))()
+            la = LaunchArgs()
+            la.struct_size = ctypes.sizeof(LaunchArgs)
+            la.value_inputs = ctypes.cast(st.v_arr, ctypes.POINTER(ctypes.c_void_p))
+            la.num_value_inputs = nv
+            la.index_inputs = ctypes.cast(st.i_arr, ctypes.POINTER(ctypes.c_void_p))
+            la.num_index_inputs = ni
+            la.outputs = ctypes.cast(st.o_arr, ctypes.POINTER(ctypes.c_void_p))
+            la.num_outputs = no
+            st.la = la
+            st.ref = ctypes.byref(la)
+            self._tls.state = st
+        return st
+
     def merged_spmv_launch(self, *args, **kwargs):
         import torch
         b = self._bind(args, kwargs)
-        values = [b[n] for n in self._value_names]
-        indices = [b[n] for n in self._index_names]
+        value_names, index_names = self._value_names, self._index_names
+        values = [b[n] for n in value_names]
+        indices = [b[n] for n in index_names]
         ro = b["row_end_offsets"]
         num_rows, num_cols = int(b["num_rows"]), int(b["num_cols"])
 
-        dispatch = b[self.signature["dispatch_tensor"]]
+        dispatch = b[self._dispatch_name]
         _check(dispatch.is_cuda, "CUDA device required")
-        for n in self._value_names + self._index_names + ["row_end_offsets"]:
+        for n in self._tensor_names:
             t = b[n]
-            _check(t.is_cuda, f"{n} must be a CUDA tensor")
-            _check(t.is_contiguous(), f"{n} must be contiguous")
-        names = {torch.float32: "float32", torch.float64: "float64", torch.int64: "int64"}
-        dt = names.get(dispatch.dtype)
+            if not t.is_cuda:
+                raise RuntimeError(f"{n} must be a CUDA tensor")
+            if not t.is_contiguous():
+                raise RuntimeError(f"{n} must be contiguous")
+        dtype = dispatch.dtype
+        dt = _TORCH_DTYPE_NAMES().get(dtype)
         _check(dt is not None and dt in self._dtypes and (dt != "int64" or self.signature["allow_int64"]),
                "Unsupported dtype for ValueT. Use float32 or float64.")
-        for n, t in zip(self._value_names, values):
-            _check(t.dtype == dispatch.dtype, f"{n} dtype mismatch")
-        for n, t in zip(self._index_names, indices):
-            _check(t.dtype == torch.int32, f"{n} dtype mismatch")
-        _check(ro.dtype == torch.int32, "row_end_offsets dtype mismatch")
+        for n, t in zip(value_names, values):
+            if t.dtype != dtype:
+                raise RuntimeError(f"{n} dtype mismatch")
+        int32 = torch.int32
+        for n, t in zip(index_names, indices):
+            if t.dtype != int32:
+                raise RuntimeError(f"{n} dtype mismatch")
+        _check(ro.dtype == int32, "row_end_offsets dtype mismatch")
 
         ne = int(indices[0].numel()) if indices else num_cols
         _check(ne > 0, "selector index must be non-empty")
-        for n, t in zip(self._index_names, indices):
-            _check(t.numel() == ne, f"{n} must have ne = {ne} entries")
-        dims = self.signature["value_dims"]
-        for n, t in zip(self._value_names, values):
-            _check(t.numel() % dims[n] == 0, f"{n}.numel() must be a multiple of its item width {dims[n]}")
+        for n, t in zip(index_names, indices):
+            if t.numel() != ne:
+                raise RuntimeError(f"{n} must have ne = {ne} entries")
+        dims = self._dims
+        for n, t in zip(value_names, values):
+            d = dims[n]
+            count = t.numel()
+            if count % d != 0:
+                raise RuntimeError(f"{n}.numel() must be a multiple of its item width {d}")
             # the kernels index a streamed tensor by edge id: a shorter one would be read out of bounds
-            if n in self._streamed:
-                _check(t.numel() >= ne * dims[n], f"{n} must hold one item of width {dims[n]} per edge ({ne})")
-        if self._has_reducer:
-            _check(ro.numel() == num_rows + 1, "row_end_offsets must have length num_rows + 1")
-            _check(num_rows + ne < 2 ** 31, "num_rows + ne must stay below 2^31 (32-bit offsets)")
+            if n in self._streamed and count < ne * d:
+                raise RuntimeError(f"{n} must hold one item of width {d} per edge ({ne})")
             # a source gathered through a row-aligned selector is read at every row id of a tile, empty
             # rows included: a tensor shorter than num_rows would be read out of bounds
-            for n, t in zip(self._value_names, values):
-                if n in self._row_indexed:
-                    _check(t.numel() >= num_rows * dims[n],
-                           f"{n} must hold one item of width {dims[n]} per row ({num_rows}): it is gathered "
-                           f"through a selector declared equal to the reducer's row ids")
+            if n in self._row_indexed and count < num_rows * d and num_rows + ne < 2 ** 31:
+                raise RuntimeError(f"{n} must hold one item of width {d} per row ({num_rows}): it is gathered "
+                                   f"through a selector declared equal to the reducer's row ids")
+        if self._has_reducer:
+            _check(ro.numel() == num_rows + 1, "row_end_offsets must have length num_rows + 1")
             if self.verify_row_aligned and self._row_aligned:
                 row_ids = torch.repeat_interleave(torch.arange(num_rows, device=ro.device, dtype=torch.int32),
                                                   (ro[1:] - ro[:-1]).to(torch.int64))
-                for n, t in zip(self._index_names, indices):
+                for n, t in zip(index_names, indices):
                     if n in self._row_aligned:
                         _check(bool(torch.equal(t, row_ids)), f"{n} was declared equal to the reducer's row ids "
                                                               f"(row_aligned) but differs from them")
 
         device = dispatch.device
         outs = []
-        for o in self._outputs:
-            lead = {"reducer": num_rows, "sum": None, "map": ne}[o["kind"]]
-            if lead is None:
-                shape = (o["dim"],)
+        for kind, dim in self._out_specs:
+            if kind == "sum":
+                shape = (dim,)
             else:
-                shape = (lead,) if o["dim"] == 1 else (lead, o["dim"])
-            outs.append(torch.empty(shape, dtype=dispatch.dtype, device=device))
+                lead = num_rows if kind == "reducer" else ne
+                shape = (lead,) if dim == 1 else (lead, dim)
+            outs.append(torch.empty(shape, dtype=dtype, device=device))
 
-        ws_bytes = self.workspace_bytes(dt, num_rows, ne)
-        stream = torch.cuda.current_stream(device)
-        ws = self._scratch(device, stream, ws_bytes)
+        size_key = (dt, num_rows, ne)
+        ws_bytes = self._ws_bytes.get(size_key)
+        if ws_bytes is None:
+            ws_bytes = self._ws_bytes[size_key] = self.workspace_bytes(dt, num_rows, ne)
+        index = device.index
+        other_device = index is not None and index != torch._C._cuda_getDevice()
+        if other_device:
+            with torch.cuda.device(device):
+                return self._launch(values, indices, outs, ro, num_rows, num_cols, ne, dt, device, index, ws_bytes)
+        return self._launch(values, indices, outs, ro, num_rows, num_cols, ne, dt, device,
+                            index if index is not None else torch._C._cuda_getDevice(), ws_bytes)
 
-        def ptr_array(tensors):
-            arr = (ctypes.c_void_p * max(len(tensors), 1))()
-            for i, t in enumerate(tensors):
-                arr[i] = t.data_ptr()
-            return arr
-
-        v_arr, i_arr, o_arr = ptr_array(values), ptr_array(indices), ptr_array(outs)
-        la = LaunchArgs()
-        la.struct_size = ctypes.sizeof(LaunchArgs)
+    def _launch(self, values, indices, outs, ro, num_rows, num_cols, ne, dt, device, index, ws_bytes):
+        """Fill the argument block and call the library on the current stream of the (current) device."""
+        import torch
+        raw_stream = torch._C._cuda_getCurrentRawStream(index)
+        ws = self._scratch(device, index, raw_stream, ws_bytes)
+        st = self._call_state()
+        la = st.la
+        for i, t in enumerate(values):
+            st.v_arr[i] = t.data_ptr()
+        for i, t in enumerate(indices):
+            st.i_arr[i] = t.data_ptr()
+        for i, t in enumerate(outs):
+            st.o_arr[i] = t.data_ptr()
         la.dtype = DTYPE_CODES[dt]
-        la.value_inputs = ctypes.cast(v_arr, ctypes.POINTER(ctypes.c_void_p))
-        la.num_value_inputs = len(values)
-        la.index_inputs = ctypes.cast(i_arr, ctypes.POINTER(ctypes.c_void_p))
-        la.num_index_inputs = len(indices)
-        la.outputs = ctypes.cast(o_arr, ctypes.POINTER(ctypes.c_void_p))
-        la.num_outputs = len(outs)
         la.row_end_offsets = ro.data_ptr()
         la.num_rows, la.num_cols, la.ne = num_rows, num_cols, ne
         la.workspace, la.workspace_bytes = ws.data_ptr(), ws.numel()
-        la.flags = (FLAG_TIME_KERNEL if self.time_kernel else 0) | int(self.extra_flags)
+        flags = (FLAG_TIME_KERNEL if self.time_kernel else 0) | int(self.extra_flags)
         if self.reuse_tiles and self._has_reducer:
-            key = (ro.data_ptr(), ro._version, num_rows, ne, dt, ws.data_ptr(), str(device))
+            key = (ro.data_ptr(), ro._version, num_rows, ne, dt, ws.data_ptr(), index)
             if key == self._tile_key:
-                la.flags |= FLAG_REUSE_TILES
+                flags |= FLAG_REUSE_TILES
             self._tile_key = key
-        with torch.cuda.device(device):
-            la.stream = stream.cuda_stream
-            rc = self._lib.flexspmv_launch(ctypes.byref(la))
+        la.flags = flags
+        la.stream = raw_stream
+        rc = self._lib.flexspmv_launch(st.ref)
         if rc != 0:
             raise RuntimeError(f"merged_spmv_launch failed ({rc}): {self._lib.flexspmv_last_error().decode()}")
         if not outs:

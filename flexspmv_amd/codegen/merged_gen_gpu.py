@@ -31,7 +31,6 @@ VERBOSE_ENV = "EASIER_VERBOSE_CODEGEN"  # same switch as the reference (codegen/
 # (160 KiB LDS per CU on gfx950).
 LDS_BUDGET_BYTES = 36 * 1024
 BLOCK_THREADS = 256
-DEFAULT_XCD_RUN = 1
 
 
 @dataclass
@@ -283,8 +282,7 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
 
     ``dtypes`` lists the value types to instantiate (default float32 + float64, plus int64 when the
     dispatch input was traced as int64 - the reference's rule, codegen/merged_gen_binding.py:143-157).
-    ``policy`` may override ``block``, ``ipt_f32``, ``ipt_f64``, ``ipt_flat`` and ``xcd_run`` (consecutive
-    tiles handed to one XCD; 1 = round-robin).
+    ``policy`` may override ``block``, ``ipt_f32``, ``ipt_f64`` and ``ipt_flat``.
     """
     inputs, outputs, selector_register, map_ops, red_ops, agg_ops = ir.six()
     kp = analyse(ir)
@@ -300,7 +298,6 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
            "int64": int(policy.get("ipt_f64", _choose_ipt(kp, 8)))}
     if not has_reducer:
         ipt = {k: int(policy.get("ipt_flat", 8)) for k in ipt}
-    xcd_run = int(policy.get("xcd_run", DEFAULT_XCD_RUN))
 
     # ---- Params ---------------------------------------------------------------------------
     params, fill = [], []
@@ -420,7 +417,7 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         # value tensors read at index `row` for every row of a tile (served from the merge path): they
         # must hold at least num_rows items
         "row_indexed_value_inputs": sorted({src for _, src, _, _ in kp.row_sources}),
-        "policy": {"block": block, "ipt": {k: ipt[k] for k in dtypes}, "xcd_run": xcd_run},
+        "policy": {"block": block, "ipt": {k: ipt[k] for k in dtypes}},
         "widths": {"exchange": kp.xch_width, "reduce": kp.red_width, "aggregate": kp.agg_width,
                    "row": kp.row_width},
     })
@@ -441,9 +438,6 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
 
     src = f"""// Generated by flexspmv_amd.codegen.merged_gen_gpu for sub-graph "{ir.name}" ({ir.content_hash()}).
 // Do not edit: regenerate from the six-list description instead.
-#ifndef FLEX_TUNE_XCD_RUN
-#define FLEX_TUNE_XCD_RUN {xcd_run}
-#endif
 #include "flex_dispatch.hpp"
 
 namespace {{

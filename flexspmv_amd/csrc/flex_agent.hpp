@@ -25,8 +25,8 @@
 //   * aggregators are block partials + one ordered final sum instead of floating-point atomics;
 //   * a reducer and an aggregator can share one pass over the edges;
 //   * one small independent block per tile; block b takes tile b, so the 8 XCDs (one L2 each, workgroups
-//     are dealt to them round-robin) work side by side on neighbouring tiles.  Longer runs of tiles per
-//     XCD cut the re-fetching of gathered data but measured no faster (tuning switch FLEX_TUNE_XCD_RUN).
+//     are dealt to them round-robin) work side by side on neighbouring tiles, in runs of 1 or 16 tiles
+//     per XCD (tile_of_block).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -112,6 +112,7 @@ struct Tiling {
   int nominal;     // merge items between two diagonals
   int snap_slack;  // 0: boundaries stay on their diagonals
   int snap_mask;   // rows per output line - 1 (power of two - 1)
+  int xcd_shift;   // runs of 2^xcd_shift consecutive tiles share an XCD (see tile_of_block)
 };
 
 __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end, int num_rows,
@@ -131,6 +132,92 @@ __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int
   return c;
 }
 
+// The same boundary found by a whole wavefront (all 64 lanes must call it; the result is uniform).
+// A search by one lane is a chain of dependent loads; here a round is one load per lane.  Up to three
+// rounds probe 64 consecutive rows around a guess: first the interpolated position, then that position
+// corrected by the residual at the edge of the window just probed (a Newton step with a 64-row
+// window).  Regular matrices end after one round, smoothly varying ones after two.  If that fails the
+// bracket shrinks 64-fold per round.  The row-start load of a snapped boundary is served from the
+// probes of the round that found the answer when that row is among them.  Result: identical to
+// tile_boundary (same monotone predicate, same rule).
+__device__ __forceinline__ int2 wave_tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end,
+                                                   int num_rows, int nnz) {
+  constexpr int LEAD = 40;  // rows of the window below the guess (covers the row a snap moves back to)
+  const int lane = lane_id();
+  const long long d = (long long)t * tl.nominal;
+  const int diag = (int)min(d, (long long)num_rows + nnz);
+  int lo = max(diag - nnz, 0);
+  int hi = min(diag, num_rows);
+  // the answer: first i in [lo, hi) with row_end[i] + i + 1 > diag, else hi
+  const float inv_slope = (float)num_rows / ((float)num_rows + (float)nnz);
+  int guess = (int)((float)diag * inv_slope);
+  int win_start = 0, win_end_value = 0;  // window of the round that found the answer, and this lane's probe
+  bool win_valid = false;
+#pragma unroll 1
+  for (int round = 0; round < 3 && lo < hi; ++round) {
+    const int w0 = min(max(guess - LEAD, lo), max(hi - WAVE, lo));  // window [w0, w0 + 64) inside [lo, hi)
+    const int pos = w0 + lane;
+    int end = 0;
+    bool past = true;  // lanes at or beyond hi behave like "predicate true"
+    if (pos < hi) {
+      end = row_end[pos];
+      past = end + pos + 1 > diag;
+    }
+    const unsigned long long m = __builtin_amdgcn_ballot_w64(past);
+    if (m == 0ull) {  // every probed row ends before the diagonal: the answer lies beyond the window
+      const int g_last = __builtin_amdgcn_readlane(end, WAVE - 1) + (w0 + WAVE - 1) + 1;
+      lo = w0 + WAVE;
+      guess = (int)min((long long)lo + (long long)((float)(diag - g_last) * inv_slope), (long long)hi);
+    } else {
+      const int j = __builtin_ctzll(m);
+      if (j > 0 || w0 == lo) {  // rows before w0 + j end before the diagonal, row w0 + j (or hi) does not
+        lo = hi = w0 + j;
+        win_start = w0;
+        win_end_value = end;
+        win_valid = true;
+      } else {  // the answer is at or before the window's first row
+        const int g_first = __builtin_amdgcn_readlane(end, 0) + w0 + 1;
+        hi = w0;
+        guess = w0 - 1 - (int)((float)(g_first - diag) * inv_slope);
+      }
+    }
+    lo = __builtin_amdgcn_readfirstlane(lo);  // uniform by construction; tell the compiler
+    hi = __builtin_amdgcn_readfirstlane(hi);
+    guess = __builtin_amdgcn_readfirstlane(guess);
+  }
+  const int probed_below = min(diag, num_rows);  // window lanes at or beyond this row hold no probe
+#pragma unroll 1
+  while (lo < hi) {  // 64 evenly spaced probes per round
+    const int n = hi - lo;
+    const int step = (n + WAVE - 1) / WAVE;
+    const int pos = lo + (lane + 1) * step - 1;
+    bool past = true;
+    if (pos < hi) past = row_end[pos] + pos + 1 > diag;
+    const unsigned long long m = __builtin_amdgcn_ballot_w64(past);
+    const int j = (m == 0ull) ? WAVE : __builtin_ctzll(m);
+    // samples before j end before the diagonal, sample j (if any) does not
+    const int new_lo = min(lo + j * step, hi);                                    // one past sample j - 1
+    const int new_hi = (j == WAVE) ? hi : min(lo + (j + 1) * step - 1, hi);      // sample j itself (or hi)
+    lo = __builtin_amdgcn_readfirstlane(new_lo);
+    hi = __builtin_amdgcn_readfirstlane(new_hi);
+  }
+  int2 c = make_int2(min(lo, num_rows), diag - lo);
+  if (tl.snap_slack > 0 && t > 0 && t < tl.num_tiles) {
+    const int xs = c.x & ~tl.snap_mask;
+    int ys = 0;
+    if (xs > 0) {
+      const int src = xs - 1 - win_start;  // lane that probed row xs - 1
+      if (win_valid && src >= 0 && src < WAVE && xs - 1 < probed_below) {
+        ys = __builtin_amdgcn_readfirstlane(__builtin_amdgcn_ds_bpermute(src << 2, win_end_value));
+      } else {
+        ys = row_end[xs - 1];
+      }
+    }
+    if ((c.x - xs) + (c.y - ys) <= tl.snap_slack) c = make_int2(xs, ys);
+  }
+  return c;
+}
+
 // One search per tile boundary: coords[t] is where tile t starts, coords[num_tiles] where the path ends.
 __global__ void __launch_bounds__(256)
 tile_search_kernel(const Tiling tl, const int* __restrict__ row_end, int num_rows, int nnz, int2* __restrict__ coords) {
@@ -140,21 +227,19 @@ tile_search_kernel(const Tiling tl, const int* __restrict__ row_end, int num_row
 }
 
 // Which tile a block works on.  Blocks are dealt to the 8 XCDs round-robin (block % 8), each XCD with
-// its own L2.  XCD_RUN consecutive tiles go to the same XCD, so that neighbouring tiles - which gather
-// overlapping vertex data - share an L2, while all XCDs still work inside one window of 8 * XCD_RUN tiles.
-#ifndef FLEX_TUNE_XCD_RUN
-#define FLEX_TUNE_XCD_RUN 1
-#endif
-constexpr int XCD_RUN = FLEX_TUNE_XCD_RUN;
-__device__ __forceinline__ int tile_of_block(int block, int num_tiles) {
-  (void)num_tiles;
-  if constexpr (XCD_RUN == 1) return block;
-  const int xcd = block % NUM_XCD, seq = block / NUM_XCD;
-  return ((seq / XCD_RUN) * NUM_XCD + xcd) * XCD_RUN + seq % XCD_RUN;
+// its own L2.  Runs of 2^xcd_shift consecutive tiles go to the same XCD, so that neighbouring tiles -
+// which gather overlapping vertex data - share an L2, while all XCDs still work inside one window of
+// 8 runs.  Runs of 16 cut the re-fetching of gathered data on meshes and stencils (Poisson 256^3: x is
+// fetched 1.2 times instead of 3.6 times) and measured 1-4 % faster there; on power-law matrices they
+// measured slower, so the host picks the run length per launch (Tiling::xcd_shift).
+__device__ __forceinline__ int tile_of_block(int block, int xcd_shift) {
+  if (xcd_shift == 0) return block;
+  const int xcd = block & (NUM_XCD - 1), seq = block / NUM_XCD;
+  return ((((seq >> xcd_shift) * NUM_XCD) + xcd) << xcd_shift) + (seq & ((1 << xcd_shift) - 1));
 }
-inline int grid_for_tiles(int num_tiles) {
-  constexpr int WINDOW = NUM_XCD * XCD_RUN;
-  return XCD_RUN == 1 ? num_tiles : (num_tiles + WINDOW - 1) / WINDOW * WINDOW;
+inline int grid_for_tiles(int num_tiles, int xcd_shift) {
+  const int window = NUM_XCD << xcd_shift;
+  return xcd_shift == 0 ? num_tiles : (num_tiles + window - 1) / window * window;
 }
 
 // ----------------------------------------------------------------------------------------------
@@ -544,8 +629,8 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
 
 // One block per tile.  The tile's coordinates come from the table tile_search_kernel wrote (coords !=
 // NULL), or - small launches, where a kernel of its own for the search costs more than the search -
-// from the block itself: lanes 0 and 1 search the two diagonals that bound the tile (the reference does
-// the same when its grid is smaller than the device, cuda_template/reducer/merged_spmv_template.cuh:97-119,
+// from the block itself: its first two wavefronts search the two diagonals that bound the tile (the
+// reference lets two threads do it when its grid is smaller than the device, cuda_template/reducer/merged_spmv_template.cuh:97-119,
 // merged_agent_spmv_template.cuh:412-435).  coords_out != NULL makes such a block leave its
 // coordinates in the table all the same (a debugging aid: the table can then be read back).
 // With FLEX_TUNE_PERSISTENT (tuning switch) a launch has at most that many blocks per CU; each walks
@@ -578,7 +663,7 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
     c1 = n1;
   }
 #else
-  const int tile = tile_of_block(blockIdx.x, num_tiles);
+  const int tile = tile_of_block(blockIdx.x, tl.xcd_shift);
   if (tile >= num_tiles) return;
   int2 c0, c1;
   if (coords != nullptr) {
@@ -586,7 +671,22 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
     c1 = coords[tile + 1];
   } else {
     __shared__ int2 s_coord[2];
-    if (threadIdx.x < 2) s_coord[threadIdx.x] = tile_boundary(tile + (int)threadIdx.x, tl, row_end, num_rows, nnz);
+    {
+      const int w = (int)threadIdx.x / WAVE;
+      if (BLOCK >= 2 * WAVE) {  // the first two wavefronts search one boundary each
+        if (w < 2) {
+          const int2 c = wave_tile_boundary(tile + w, tl, row_end, num_rows, nnz);
+          if ((threadIdx.x & (WAVE - 1)) == 0) s_coord[w] = c;
+        }
+      } else {
+        const int2 a = wave_tile_boundary(tile, tl, row_end, num_rows, nnz);
+        const int2 b = wave_tile_boundary(tile + 1, tl, row_end, num_rows, nnz);
+        if (threadIdx.x == 0) {
+          s_coord[0] = a;
+          s_coord[1] = b;
+        }
+      }
+    }
     __syncthreads();
     c0 = s_coord[0];
     c1 = s_coord[1];

@@ -115,6 +115,9 @@ inline int resident_grid(KernelT kernel, int block_threads, GridCache& cache) {
 #ifndef FLEX_TUNE_SNAP_BYTES
 #define FLEX_TUNE_SNAP_BYTES 128  // tiles start on rows whose outputs start a line of this many bytes (0: never)
 #endif
+#ifndef FLEX_TUNE_XCD_RUN_SHIFT
+#define FLEX_TUNE_XCD_RUN_SHIFT 4  // launches with row-snapped tiles hand runs of 2^4 tiles to one XCD
+#endif
 #ifndef FLEX_TUNE_INBLOCK_MAX_TILES
 #define FLEX_TUNE_INBLOCK_MAX_TILES 8192  // launches of at most this many tiles search inside the reducer blocks
 #endif
@@ -146,6 +149,7 @@ struct Dispatch {
     t.nominal = TILE;
     t.snap_slack = 0;
     t.snap_mask = 0;
+    t.xcd_shift = 0;
     if (REDUCER && FLEX_TUNE_SNAP_BYTES > 0 && num_rows > 0) {
       const int snap_rows = FLEX_TUNE_SNAP_BYTES / (int)sizeof(V) > 1 ? FLEX_TUNE_SNAP_BYTES / (int)sizeof(V) : 1;
       const int64_t slack = (snap_rows * (num_rows + ne) + num_rows - 1) / num_rows;  // snap_rows average rows
@@ -153,6 +157,7 @@ struct Dispatch {
         t.snap_slack = (int)slack;
         t.snap_mask = snap_rows - 1;
         t.nominal = TILE - (int)slack;
+        t.xcd_shift = FLEX_TUNE_XCD_RUN_SHIFT;  // short rows: neighbouring tiles gather neighbouring data
       }
     }
     const int64_t items = REDUCER ? num_rows + ne : ne;
@@ -270,7 +275,7 @@ struct Dispatch {
 #ifdef FLEX_TUNE_PERSISTENT
       const int reduce_grid = l.num_tiles < 256 * FLEX_TUNE_PERSISTENT ? l.num_tiles : 256 * FLEX_TUNE_PERSISTENT;
 #else
-      const int reduce_grid = grid_for_tiles(l.num_tiles);
+      const int reduce_grid = grid_for_tiles(l.num_tiles, l.tiling.xcd_shift);
 #endif
       const int2* table = l.search_in_blocks ? nullptr : coords;
       int2* table_out = (l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_KEEP_TILES) != 0) ? coords : nullptr;
