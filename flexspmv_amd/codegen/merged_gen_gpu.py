@@ -11,9 +11,18 @@ type ``Graph<ValueT>`` consumed by the hand-written kernels of ``csrc/flex_agent
   (codegen/merged_gen_gpu.py:188-298): ``add sub mul pow truediv neg add_ exp norm getitem clone copy_
   setitem abs sign lt gt where`` (``reducer`` / ``sum`` are routed to the reduction machinery);
 * a kernel may hold reducers AND aggregators (the reference's templates hold one or the other,
-  codegen/merged_gen_gpu.py:394);
-* ops that depend on a ``row_aligned`` selector run in the merge walk, where the row is known; the
-  values they need from the coalesced stage travel through LDS next to the reducer arguments.
+  codegen/merged_gen_gpu.py:394).
+
+What a generated ``Graph`` splits by memory level, because the kernels schedule the levels differently
+from the reference's one-statement-after-the-other body:
+
+* ``Fetch``   what is streamed per edge (edge tensors, selector indices): loaded in coalesced order and
+  handed through LDS to the thread that owns the edge's row;
+* ``Gather``  vertex data addressed through ``Fetch`` - gathered by the row's thread, so that
+  neighbouring lanes (neighbouring rows) gather neighbouring vertices;
+* ``Row``     sources of ``row_aligned`` selectors (index array == the reducer's row ids): read once
+  per row at the row id, the index array is never touched;
+* ``edge()``  the whole map for one edge: contributions to the reducers and the aggregators.
 """
 from __future__ import annotations
 
@@ -27,8 +36,8 @@ from .merged_gen_binding import BindingPlan, binding_plan, generate_binding_code
 
 VERBOSE_ENV = "EASIER_VERBOSE_CODEGEN"  # same switch as the reference (codegen/merged_gen_gpu.py:140)
 
-# LDS a reducer block may use for the per-edge exchange + row offsets; keeps >= 4 blocks per CU
-# (160 KiB LDS per CU on gfx950).
+# LDS a reducer block may use for the per-edge hand-over (keeps >= 4 blocks per CU: 160 KiB LDS per CU
+# on gfx950).
 LDS_BUDGET_BYTES = 36 * 1024
 BLOCK_THREADS = 256
 
@@ -39,20 +48,20 @@ class Var:
     kind: str          # 'tensor' | 'scalar'
     dim: int
     ctype: str         # C++ type name inside Graph<ValueT>
-    stage: int         # stage that defines it: 1 = coalesced edge stage, 2 = merge-walk stage
-    final_stage: int = 1   # stage holding its last value (an in-place op in the walk raises it)
 
 
 @dataclass
 class KernelPlan:
     plan: BindingPlan
     vars: Dict[str, Var]
-    exchange: List[Tuple[str, int, int]]      # (variable, component, slot)
-    row_sources: List[Tuple[str, str, int, int]]  # (selector var, source tensor, dim, first slot)
-    red_slices: List[Tuple[str, int, int]]    # (reducer name, first slot, dim)
+    fetch_values: List[Tuple[str, str, int, int]]     # (variable, source tensor, dim, first value slot)
+    fetch_indices: List[Tuple[str, int]]              # (selector module, index slot)
+    gathers: List[Tuple[str, str, str, int]]          # (variable, selector module, source tensor, dim)
+    row_sources: List[Tuple[str, str, int, int]]      # (selector var, source tensor, dim, first slot)
+    red_slices: List[Tuple[str, int, int]]            # (reducer name, first slot, dim)
     agg_slices: List[Tuple[str, int, int]]
-    op_stage: Dict[int, int] = field(default_factory=dict)   # index into map_operations -> stage
-    xch_width: int = 0
+    fetch_value_width: int = 0
+    fetch_index_width: int = 0
     red_width: int = 0
     agg_width: int = 0
     row_width: int = 0
@@ -69,111 +78,63 @@ def _literal(a: Any) -> str:
 
 
 def analyse(ir: FusedGraphIR) -> KernelPlan:
-    """Variable table, stage split and LDS slot assignment for a sub-graph.
-
-    A ``row_aligned`` selector may be served from the merge path (no index array read, its dependants
-    run in the walk) or like any other selector (index array read, everything runs in the coalesced
-    stage).  The first is taken only when it does not widen the per-edge LDS exchange: for ``y = A x``
-    with ``x . y`` it saves the 4-byte index per edge for free, for the mesh maps it would push every
-    input through LDS and shrink the tile.
-    """
-    with_rows = _analyse(ir, use_row_aligned=True)
-    if with_rows.row_width == 0:
-        return with_rows
-    plain = _analyse(ir, use_row_aligned=False)
-    return with_rows if with_rows.xch_width <= plain.xch_width else plain
-
-
-def _analyse(ir: FusedGraphIR, use_row_aligned: bool) -> KernelPlan:
+    """Variable table and memory-level split of a sub-graph (raises ``ValueError`` for an operation the
+    generators cannot express)."""
     inputs, outputs, selector_register, map_ops, red_ops, agg_ops = ir.six()
     plan = binding_plan(inputs, outputs, selector_register)
     has_reducer = bool(red_ops)
     vars: Dict[str, Var] = {}
-
-    cur_stage: Dict[str, int] = {}   # stage a variable's current value lives in (in-place ops may raise it)
+    fetch_values: List[Tuple[str, str, int, int]] = []
+    fetch_indices: List[Tuple[str, int]] = []
+    gathers: List[Tuple[str, str, str, int]] = []
+    row_sources: List[Tuple[str, str, int, int]] = []
+    value_slot = row_slot = 0
+    index_slot: Dict[str, int] = {}
     for s in selector_register:
         dim = get_dim_length(s["shape"])
-        stage = 2 if (use_row_aligned and s.get("row_aligned") and has_reducer and s["selector"] == 1) else 1
-        var = s["name"] if s["selector"] == 1 else s["selector_name"]
-        vars[var] = Var(var, "tensor", dim, f"TensorInput_{s['target']}_T", stage)
-        cur_stage[var] = stage
+        ctype = f"TensorInput_{s['target']}_T"
+        if s["selector"] != 1:
+            var = s["selector_name"]
+            fetch_values.append((var, s["target"], dim, value_slot))
+            value_slot += dim
+        elif s.get("row_aligned") and has_reducer:
+            var = s["name"]
+            row_sources.append((var, s["target"], dim, row_slot))
+            row_slot += dim
+        else:
+            var = s["name"]
+            module = s["selector_name"]
+            if module not in index_slot:
+                index_slot[module] = len(fetch_indices)
+                fetch_indices.append((module, index_slot[module]))
+            gathers.append((var, module, s["target"], dim))
+        vars[var] = Var(var, "tensor", dim, ctype)
 
-    # values crossing from stage 1 into stage 2 travel through LDS slots
-    exchange: List[Tuple[str, int, int]] = []
-    slot_of: Dict[Tuple[str, int], int] = {}
-
-    def need(var: str) -> None:
-        v = vars[var]
-        for c in range(v.dim):
-            if (var, c) not in slot_of:
-                slot_of[(var, c)] = len(exchange)
-                exchange.append((var, c, len(exchange)))
-
-    # reducer arguments take the first slots so that a plain SpMV exchanges exactly its products
-    red_arg_names = [arg_name(r["args"][0]) for r in red_ops]
-
-    op_stage: Dict[int, int] = {}
-    for op_index, op in enumerate(map_ops):
+    for op in map_ops:
         o = op["op"]
-        if o in ("reducer", "sum"):
-            continue
-        args = [arg_name(a) for a in (op["args"] if o not in ("getitem", "setitem") else
-                                      [op["args"][0]] + ([op["args"][2]] if o == "setitem" else []))]
-        used = [a for a in args if isinstance(a, str) and a in vars]
-        stage = max([1] + [cur_stage[a] for a in used]) if has_reducer else 1
-        op_stage[op_index] = stage
-        if stage == 2:
-            for a in used:
-                if vars[a].stage == 1:
-                    need(a)
-        if o in ("setitem", "copy_", "add_"):
-            if o in ("setitem", "add_"):
-                cur_stage[args[0]] = max(cur_stage[args[0]], stage)
+        if o in ("reducer", "sum", "setitem", "copy_", "add_"):
             continue
         dim = get_dim_length(op["shape"])
         if o == "norm":
-            vars[op["name"]] = Var(op["name"], "scalar", 1, "ValueT", stage)
+            vars[op["name"]] = Var(op["name"], "scalar", 1, "ValueT")
         else:
-            vars[op["name"]] = Var(op["name"], "tensor", dim, f"TensorOutput_{op['name']}_T", stage)
-        cur_stage[op["name"]] = stage
+            vars[op["name"]] = Var(op["name"], "tensor", dim, f"TensorOutput_{op['name']}_T")
 
     red_slices, agg_slices = [], []
     off = 0
     for r in red_ops:
-        a = arg_name(r["args"][0])
         dim = get_dim_length(r["shape"])
         red_slices.append((r["name"], off, dim))
         off += dim
-        if vars[a].stage == 1:
-            need(a)
     red_width = off
     off = 0
     for g in agg_ops:
         dim = get_dim_length(g["shape"])
         agg_slices.append((g["name"], off, dim))
         off += dim
-    agg_width = off
-    for g in agg_ops:
-        a = arg_name(g["args"][0])
-        if has_reducer and cur_stage[a] == 2 and vars[a].stage == 1:
-            need(a)
-    # put reducer-argument slots first (stable order otherwise)
-    order = sorted(range(len(exchange)), key=lambda i: (exchange[i][0] not in red_arg_names, i))
-    exchange = [(exchange[i][0], exchange[i][1], n) for n, i in enumerate(order)]
-    for var in vars:
-        vars[var].final_stage = cur_stage[var]
-
-    row_sources: List[Tuple[str, str, int, int]] = []
-    row_width = 0
-    for s in selector_register:
-        if s["selector"] == 1 and vars[s["name"]].stage == 2 and s.get("row_aligned") and use_row_aligned:
-            dim = get_dim_length(s["shape"])
-            row_sources.append((s["name"], s["target"], dim, row_width))
-            row_width += dim
-
-    return KernelPlan(plan, vars, exchange, row_sources, red_slices, agg_slices, op_stage=op_stage,
-                      xch_width=len(exchange), red_width=red_width, agg_width=agg_width,
-                      row_width=row_width)
+    return KernelPlan(plan, vars, fetch_values, fetch_indices, gathers, row_sources, red_slices, agg_slices,
+                      fetch_value_width=value_slot, fetch_index_width=len(fetch_indices), red_width=red_width,
+                      agg_width=off, row_width=row_slot)
 
 
 # ------------------------------------------------------------------------------------------
@@ -182,26 +143,6 @@ def _analyse(ir: FusedGraphIR, use_row_aligned: bool) -> KernelPlan:
 def _arg(a: Any) -> str:
     a = arg_name(a)
     return a if isinstance(a, str) else _literal(a)
-
-
-def _emit_selector(s: Dict[str, Any]) -> Tuple[List[str], List[str], List[str], List[str], List[str]]:
-    """Statements of one stage-1 selector entry, split by memory level:
-    (Fetch members, fetch statements, Gather members, gather statements, stage-1 prologue)."""
-    dim = get_dim_length(s["shape"])
-    T = f"TensorInput_{s['target']}_T"
-    if s["selector"] == 1:
-        name, idx = s["name"], f"column_indices_{s['name']}"
-        return ([f"OffsetT {idx};"],
-                [f"q_f.{idx} = flex::stream_load(q_p.{s['selector_name']}_idx_ptr + q_e);"],
-                [f"{T} {name};"],
-                [f"q_g.{name} = {T}(q_p.{s['target']}_ptr + (size_t)q_f.{idx} * {dim});"],
-                [f"{T} {name} = q_g.{name};"])
-    name = s["selector_name"]
-    return ([f"{T} {name};"],
-            [f"q_f.{name}.values[{i}] = flex::stream_load(q_p.{s['target']}_ptr + (size_t)q_e * {dim} + {i});"
-             for i in range(dim)],
-            [], [],
-            [f"{T} {name} = q_f.{name};"])
 
 
 def _store_loop(ptr: str, edge: str, dim: int, src: str, src_dim: int) -> List[str]:
@@ -268,8 +209,8 @@ def _indent(lines: Sequence[str], n: int = 4) -> str:
 
 def _choose_ipt(kp: KernelPlan, value_bytes: int) -> int:
     """Items per thread so that one block's LDS stays inside LDS_BUDGET_BYTES."""
-    # LDS holds the per-edge exchange of a tile and, in the merge path, one finished total per row
-    per_item = value_bytes * max(kp.xch_width, kp.red_width, 1)
+    # LDS holds what is fetched per edge of a tile and, in the merge path, one finished total per row
+    per_item = max(value_bytes * kp.fetch_value_width + 4 * kp.fetch_index_width, value_bytes * kp.red_width, 1)
     for ipt in (8, 4, 2, 1):
         if BLOCK_THREADS * ipt * per_item <= LDS_BUDGET_BYTES:
             return ipt
@@ -321,41 +262,38 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         if op["op"] not in ("reducer", "sum", "norm", "setitem", "copy_", "add_"):
             typedefs.append(f"typedef flex::Tensor<ValueT, {get_dim_length(op['shape'])}> TensorOutput_{op['name']}_T;")
 
-    # ---- stage bodies ---------------------------------------------------------------------
-    s1: List[str] = []
-    s2: List[str] = []
-    fetch_members: List[str] = []
-    fetch_body: List[str] = []
-    gather_members: List[str] = []
-    gather_body: List[str] = []
-    for s in selector_register:
-        var = s["name"] if s["selector"] == 1 else s["selector_name"]
-        if kp.vars[var].stage == 1:
-            fm, fs, gm, gs, pro = _emit_selector(s)
-            fetch_members += fm
-            fetch_body += fs
-            gather_members += gm
-            gather_body += gs
-            s1 += pro
-    # rebuild crossing variables and row-aligned selector values at the top of stage 2
-    rebuilt = set()
-    for var, c, slot in kp.exchange:
-        v = kp.vars[var]
-        if var not in rebuilt:
-            s2.append(f"{v.ctype} {var};" if v.kind == "tensor" else f"ValueT {var};")
-            rebuilt.add(var)
-        s2.append(f"{_component(v, c)} = q_xch.v[{slot}];")
-    for sel, src, dim, first in kp.row_sources:
-        s2.append(f"TensorInput_{src}_T {sel};")
-        s2 += [f"{sel}.values[{i}] = q_rv.v[{first + i}];" for i in range(dim)]
+    # ---- memory levels --------------------------------------------------------------------
+    fetch_members, fetch_body, put_body, get_body = [], [], [], []
+    gather_members, gather_body = [], []
+    body: List[str] = []          # edge(): prologue, map operations, reducer / aggregator arguments
+    for var, target, dim, first in kp.fetch_values:
+        T = kp.vars[var].ctype
+        fetch_members.append(f"{T} {var};")
+        fetch_body += [f"q_f.{var}.values[{i}] = flex::stream_load(q_p.{target}_ptr + (size_t)q_e * {dim} + {i});"
+                       for i in range(dim)]
+        put_body += [f"q_sv[{first + i} * TILE + q_j] = q_f.{var}.values[{i}];" for i in range(dim)]
+        get_body += [f"q_f.{var}.values[{i}] = q_sv[{first + i} * TILE + q_j];" for i in range(dim)]
+        body.append(f"{T} {var} = q_f.{var};")
+    for module, slot in kp.fetch_indices:
+        fetch_members.append(f"OffsetT index_{module};")
+        fetch_body.append(f"q_f.index_{module} = flex::stream_load(q_p.{module}_idx_ptr + q_e);")
+        put_body.append(f"q_si[{slot} * TILE + q_j] = q_f.index_{module};")
+        get_body.append(f"q_f.index_{module} = q_si[{slot} * TILE + q_j];")
+    for var, module, target, dim in kp.gathers:
+        T = kp.vars[var].ctype
+        gather_members.append(f"{T} {var};")
+        gather_body.append(f"q_g.{var} = {T}(q_p.{target}_ptr + (size_t)q_f.index_{module} * {dim});")
+        body.append(f"{T} {var} = q_g.{var};")
+    load_row = []
+    for var, target, dim, first in kp.row_sources:
+        load_row += [f"q_rv.v[{first + i}] = q_p.{target}_ptr[(size_t)q_row * {dim} + {i}];" for i in range(dim)]
+        body.append(f"{kp.vars[var].ctype} {var};")
+        body += [f"{var}.values[{i}] = q_rv.v[{first + i}];" for i in range(dim)]
 
     map_output_names = {o.name: o for o in plan.outputs if o.kind == "map"}
-    for op_index, op in enumerate(map_ops):
-        o = op["op"]
-        if o in ("reducer", "sum"):
+    for op in map_ops:
+        if op["op"] in ("reducer", "sum"):
             continue
-        stage = kp.op_stage.get(op_index, 1) if has_reducer else 1
-        body = s1 if stage == 1 else s2
         body.extend(_emit_map(op, kp.vars, "q_e"))
         if op["name"] in map_output_names:
             out = map_output_names[op["name"]]
@@ -364,41 +302,20 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
                 body.append(f"flex::stream_store(q_p.output_y_{out.name}_ptr + (size_t)q_e, {v.name});")
             else:
                 body.extend(_store_loop(f"q_p.output_y_{out.name}_ptr", "q_e", out.dim, v.name, v.dim))
-    # a map output may also be a (stage-1) selector / input variable
+    # a map output may also be a selector / input variable
     for name, out in map_output_names.items():
         if not any(op["name"] == name for op in map_ops):
             v = kp.vars[name]
-            (s1 if v.stage == 1 or not has_reducer else s2).extend(
-                _store_loop(f"q_p.output_y_{out.name}_ptr", "q_e", out.dim, v.name, v.dim))
-
-    agg2_mask = 0
-    stage1_has_agg = False
-    # reducer arguments
+            body.extend(_store_loop(f"q_p.output_y_{out.name}_ptr", "q_e", out.dim, v.name, v.dim))
     for (rname, first, dim), r in zip(kp.red_slices, red_ops):
         v = kp.vars[arg_name(r["args"][0])]
-        for c in range(dim):
-            s2.append(f"q_tot.v[{first + c}] = {_component(v, c % v.dim)};")
-    # aggregator arguments
+        body += [f"q_tot.v[{first + c}] = {_component(v, c % v.dim)};" for c in range(dim)]
     for (gname, first, dim), g in zip(kp.agg_slices, agg_ops):
         v = kp.vars[arg_name(g["args"][0])]
-        in_walk = has_reducer and v.final_stage == 2
-        for c in range(dim):
-            if in_walk:
-                s2.append(f"q_agg.v[{first + c}] = {_component(v, c % v.dim)};")
-                agg2_mask |= 1 << (first + c)
-            else:
-                s1.append(f"q_agg.v[{first + c}] += {_component(v, c % v.dim)};")
-                stage1_has_agg = True
-    # exchange writes close stage 1
-    if has_reducer:
-        for var, c, slot in kp.exchange:
-            s1.append(f"q_xch.v[{slot}] = {_component(kp.vars[var], c)};")
+        body += [f"q_agg.v[{first + c}] = {_component(v, c % v.dim)};" for c in range(dim)]
+    edge_pure = not any("stream_store(" in line for line in body)
 
-    stage2_pure = not any("stream_store(" in line for line in s2)
-    stage1_pure = not stage1_has_agg and not any("stream_store(" in line for line in s1)
-    load_row, store_row, add_row, store_agg = [], [], [], []
-    for sel, src, dim, first in kp.row_sources:
-        load_row += [f"q_rv.v[{first + i}] = q_p.{src}_ptr[(size_t)q_row * {dim} + {i}];" for i in range(dim)]
+    store_row, add_row, store_agg = [], [], []
     for (rname, first, dim) in kp.red_slices:
         for c in range(dim):
             store_row.append(f"flex::stream_store(q_p.output_y_{rname}_ptr + (size_t)q_row * {dim} + {c}, q_tot.v[{first + c}]);")
@@ -407,19 +324,21 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         for c in range(dim):
             store_agg.append(f"q_p.output_y_{gname}_ptr[{c}] = q_total.v[{first + c}];")
 
+    row_aligned_modules = sorted({s["selector_name"] for s in selector_register
+                                  if s["selector"] == 1 and s.get("row_aligned") and has_reducer})
+    read_modules = {module for module, _ in kp.fetch_indices}
     signature = generate_binding_code(None, inputs, outputs, selector_register)
     signature.update({
         "graph": ir.name,
         "hash": ir.content_hash(),
         "dtypes": list(dtypes),
-        "row_aligned_index_inputs": sorted({s["selector_name"] + "_idx" for s in selector_register
-                                            if s["selector"] == 1 and kp.vars[s["name"]].stage == 2}),
-        # value tensors read at index `row` for every row of a tile (served from the merge path): they
-        # must hold at least num_rows items
+        # index arrays the library never dereferences: their selector equals the reducer's row ids
+        "row_aligned_index_inputs": [m + "_idx" for m in row_aligned_modules if m not in read_modules],
+        # value tensors read at index `row` for every row of a tile: they must hold at least num_rows items
         "row_indexed_value_inputs": sorted({src for _, src, _, _ in kp.row_sources}),
         "policy": {"block": block, "ipt": {k: ipt[k] for k in dtypes}},
-        "widths": {"exchange": kp.xch_width, "reduce": kp.red_width, "aggregate": kp.agg_width,
-                   "row": kp.row_width},
+        "widths": {"fetch_values": kp.fetch_value_width, "fetch_indices": kp.fetch_index_width,
+                   "reduce": kp.red_width, "aggregate": kp.agg_width, "row": kp.row_width},
     })
     sig_json = json.dumps(signature, sort_keys=True)
     sig_literal = json.dumps(sig_json)  # a C string literal
@@ -446,16 +365,16 @@ template <typename ValueT>
 struct Graph {{
   using Value = ValueT;
   using OffsetT = int;
-  static constexpr int XCH_WIDTH = {kp.xch_width};
+  static constexpr int FETCH_VALUES = {kp.fetch_value_width};   // ValueT words streamed per edge
+  static constexpr int FETCH_INDICES = {kp.fetch_index_width};  // index words streamed per edge
   static constexpr int RED_WIDTH = {kp.red_width};
   static constexpr int AGG_WIDTH = {kp.agg_width};
   static constexpr int ROW_WIDTH = {kp.row_width};
-  // stage 2 has no side effects besides its accumulators, so the walk may run it unconditionally
-  static constexpr bool STAGE2_PURE = {'true' if stage2_pure else 'false'};
-  // likewise stage 1 (no stores, no aggregator fed from the coalesced stage)
-  static constexpr bool STAGE1_PURE = {'true' if stage1_pure else 'false'};
-  // aggregator slots fed from the merge walk (the others are summed in stage 1)
-  static constexpr unsigned AGG2_MASK = {agg2_mask}u;
+  // 32-bit registers that hold one edge's fetched and gathered data
+  static constexpr int EDGE_WORDS = ({kp.fetch_value_width} + {sum(d for _, _, _, d in kp.gathers)}) * (int)(sizeof(ValueT) / 4) + {kp.fetch_index_width};
+  // edge() has no side effects besides its results, so a kernel may evaluate it for a lane that has no
+  // edge and discard the result
+  static constexpr bool EDGE_PURE = {'true' if edge_pure else 'false'};
 
   struct Params {{
 {_indent(params)}  }};
@@ -474,17 +393,19 @@ struct Graph {{
 {_indent(fetch_body)}  }}
   static FLEX_DEV void gather(const Params& q_p, const Fetch& q_f, Gather& q_g) {{
 {_indent(gather_body)}  }}
+  // hand-over of a tile's fetched data through LDS: word w of tile edge j sits at [w * TILE + j]
+  template <int TILE>
+  static FLEX_DEV void put(const Fetch& q_f, ValueT* q_sv, OffsetT* q_si, const int q_j) {{
+{_indent(put_body)}  }}
+  template <int TILE>
+  static FLEX_DEV void get(const ValueT* q_sv, const OffsetT* q_si, const int q_j, Fetch& q_f) {{
+{_indent(get_body)}  }}
 
-  // coalesced edge stage: the map on fetched + gathered data
-  template <class X, class A>
-  static FLEX_DEV void stage1(const Params& q_p, const int q_e, const Fetch& q_f, const Gather& q_g, X& q_xch, A& q_agg) {{
-{_indent(s1)}  }}
-
-  // merge-walk stage (row known): what edge e contributes to the reducers (tot) and to the
-  // aggregators fed from the walk (agg); both are assigned, the kernel accumulates
-  template <class X, class R, class T, class A>
-  static FLEX_DEV void contrib(const Params& q_p, const int q_e, const int q_row, const X& q_xch, const R& q_rv, T& q_tot, A& q_agg) {{
-{_indent(s2)}  }}
+  // the map for edge q_e: what it contributes to the reducers (q_tot) and to the aggregators (q_agg);
+  // both are assigned, the kernel accumulates
+  template <class R, class T, class A>
+  static FLEX_DEV void edge(const Params& q_p, const int q_e, const Fetch& q_f, const Gather& q_g, const R& q_rv, T& q_tot, A& q_agg) {{
+{_indent(body)}  }}
 
   template <class R>
   static FLEX_DEV void load_row(const Params& q_p, const int q_row, R& q_rv) {{
@@ -545,10 +466,8 @@ int flexspmv_launch_static(const flexspmv_launch_args* a) {{
 }}  // extern "C"
 """
     if os.getenv(VERBOSE_ENV) in ("1", "", "true", "True"):
-        for line in s1:
-            print("Stage-1 code: ", line)
-        for line in s2:
-            print("Stage-2 code: ", line)
+        for line in body:
+            print("Edge code: ", line)
     return src, signature
 
 

@@ -3,11 +3,11 @@
 // A generated translation unit defines a graph type G (see codegen/merged_gen_gpu.py) and instantiates
 // the kernels below with it.  G supplies, for value type V:
 //   G::Params                      pointer bundle (kernel argument)
-//   XCH / RED / AGG / ROW widths   number of V values per edge passed through LDS, per-row reduced,
-//                                  globally summed, and staged per tile row
+//   FETCH_VALUES / FETCH_INDICES   V words and index words streamed per edge (handed through LDS)
+//   RED / AGG / ROW widths         number of V values per-row reduced, globally summed, and read per row
 //   fetch / gather                 first-level (streamed) and second-level (gathered) loads of edge e
-//   stage1(p, e, f, g, xch, agg)   the map for edge e in coalesced order; fills xch, adds to agg
-//   contrib(p, e, row, xch, rv, tot, agg)  the part of the map that needs the row; assigns tot / agg
+//   put / get                      a Fetch to / from its LDS slot
+//   edge(p, e, f, g, rv, tot, agg) the map for edge e; assigns its contributions tot / agg
 //   load_row / store_row / add_row / store_agg   row-aligned sources and outputs
 //
 // What the kernels replace in the reference (CUDA + CUB):
@@ -243,19 +243,22 @@ inline int grid_for_tiles(int num_tiles, int xcd_shift) {
 }
 
 // ----------------------------------------------------------------------------------------------
-// Reducer kernel.  One block per merge tile of BLOCK*IPT merge items (R row ends + Z non-zeros,
-// R + Z = BLOCK*IPT), found by the tile search kernel.  Blocks are small and independent; overlap of
-// one block's memory waits with another block's arithmetic is left to the hardware scheduler (7-8
-// resident blocks per CU), which measured far better than a persistent, software-pipelined loop.
+// Reducer kernel.  One block per merge tile of at most BLOCK*IPT merge items (R row ends + Z non-zeros),
+// found by the tile search.  Blocks are small and independent; overlap of one block's memory waits
+// with another block's arithmetic is left to the hardware scheduler (6-8 resident blocks per CU), which
+// measured far better than a persistent, software-pipelined loop.
 //
 //   1  first-level loads: IPT edges per thread in coalesced order (edge tensors, index arrays), the
 //      end offset of tile row tid (first wavefront: also of row BLOCK + tid) and row-aligned sources
-//   2  second-level loads: gathers through the index arrays
-//   3  the map runs in coalesced edge order; per-edge values needed per row go to LDS
-//   4  a block-wide vote picks the reduction:
-//      ROW path (every row of the tile has at most ROW_PATH_MAX_LEN non-zeros - meshes, stencils):
-//        thread r owns tile row r, sums its products from LDS and stores the result; consecutive
-//        threads write consecutive rows.  Book-keeping is per row, not per item.
+//   2  what was fetched goes to LDS; a block-wide vote (which doubles as the barrier that publishes
+//      the LDS data) picks the reduction:
+//      ROW path (every row of the tile is short and about as long as its neighbours - meshes,
+//        stencils): thread r owns tile row r.  It takes the row's edges from LDS, gathers their vertex
+//        data, runs the map and sums.  Neighbouring lanes are neighbouring rows, so their k-th edges
+//        point at neighbouring vertices: a wavefront's gather touches a few cache lines instead of 64
+//        (with one gather per lane in edge order the vector L1 is the limit: it looks up one line per
+//        cycle, and the 7-point stencil kept it busy 86 % of the time).  Consecutive threads store
+//        consecutive rows.
 //      MERGE path (skewed rows): each thread owns IPT consecutive merge items as in the reference
 //        (cuda_template/reducer/merged_agent_spmv_template.cuh:196-345).  Row ends become a bitmap
 //        over merge positions in LDS (row i ends at position (row_end[i] - y0) + i); a popcount
@@ -272,33 +275,46 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
             const int nnz, const typename G::Params& p, int* __restrict__ carry_row,
             typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials) {
   using V = typename G::Value;
+  using Fetch = typename G::Fetch;
+  using Gather = typename G::Gather;
   constexpr int TILE = BLOCK * IPT;
   constexpr int NW = BLOCK / WAVE;
   constexpr int NWORDS = TILE / 32;
-  constexpr int XCH = G::XCH_WIDTH, RED = G::RED_WIDTH, AGG = G::AGG_WIDTH, ROW = G::ROW_WIDTH;
+  constexpr int FV = G::FETCH_VALUES, FI = G::FETCH_INDICES;
+  constexpr int RED = G::RED_WIDTH, AGG = G::AGG_WIDTH, ROW = G::ROW_WIDTH;
   constexpr int REDN = RED > 0 ? RED : 1;
-  constexpr int XCHN = XCH > 0 ? XCH : 1;
+  constexpr int FVN = FV > 0 ? FV : 1, FIN = FI > 0 ? FI : 1;
   constexpr int OUT_CAP = TILE;               // merge path: every row a tile can finish is buffered in LDS
   constexpr int OUT_STRIDE = OUT_CAP + WAVE;  // + one dump slot per lane for items that close no row
 #ifndef FLEX_TUNE_ROW_PATH_MAX_LEN
 #define FLEX_TUNE_ROW_PATH_MAX_LEN 32
 #endif
   constexpr int ROW_PATH_MAX_LEN = FLEX_TUNE_ROW_PATH_MAX_LEN;  // longest row the row path accepts (0: never)
-  constexpr int ROW_PATH_UNROLL = 8;          // non-zeros of a row read from LDS up front
+  // Edges whose fetched and gathered data a thread keeps in registers at a time: as many as fit a budget
+  // of 32-bit registers (the shallow-water map in float64 needs 13 per edge, plain SpMV 3 to 5), so that
+  // wide graphs keep their occupancy.
+#ifndef FLEX_TUNE_STAGE_WORDS
+#define FLEX_TUNE_STAGE_WORDS 40
+#endif
+  constexpr int STAGE_FIT = FLEX_TUNE_STAGE_WORDS / (G::EDGE_WORDS > 0 ? G::EDGE_WORDS : 1);
+  constexpr int ROW_PATH_UNROLL = STAGE_FIT < 2 ? 2 : (STAGE_FIT > 8 ? 8 : STAGE_FIT);
+  constexpr int MERGE_CHUNK = ROW_PATH_UNROLL < IPT ? ROW_PATH_UNROLL : IPT;  // likewise in the merge walk
   constexpr int ROW_PATH_MAX_ROWS = BLOCK + WAVE;  // rows (incl. the open one) whose ends are prefetched
   static_assert((IPT & (IPT - 1)) == 0 && IPT <= 32, "a thread's items must sit inside one bitmap word");
   static_assert(NWORDS <= WAVE, "one wavefront scans the bitmap words");
 
-  // s_xch holds the per-edge values of the tile, s_out the rows the merge path finishes.  Where both
-  // fit a modest budget they are separate; otherwise s_out reuses s_xch after a barrier.
+  // s_fv / s_fi hold what was fetched for the tile's edges, s_out the rows the merge path finishes.
+  // Where both fit a modest budget they are separate; otherwise s_out reuses s_fv after a barrier.
 #ifndef FLEX_TUNE_SEPARATE_OUT_BYTES
 #define FLEX_TUNE_SEPARATE_OUT_BYTES (20 * 1024)
 #endif
-  constexpr int XCH_ELEMS = XCHN * TILE, OUT_ELEMS = REDN * OUT_STRIDE;
-  constexpr bool SEPARATE_OUT = (size_t)(XCH_ELEMS + OUT_ELEMS) * sizeof(V) <= (size_t)FLEX_TUNE_SEPARATE_OUT_BYTES;
-  constexpr int LDS_ELEMS = SEPARATE_OUT ? XCH_ELEMS + OUT_ELEMS : (XCH_ELEMS > OUT_ELEMS ? XCH_ELEMS : OUT_ELEMS);
-  __shared__ V s_xch[LDS_ELEMS];
-  V* const s_out = SEPARATE_OUT ? s_xch + XCH_ELEMS : s_xch;
+  constexpr int FV_ELEMS = FVN * TILE, OUT_ELEMS = REDN * OUT_STRIDE;
+  constexpr bool SEPARATE_OUT =
+      (size_t)(FV_ELEMS + OUT_ELEMS) * sizeof(V) + (size_t)FIN * TILE * 4 <= (size_t)FLEX_TUNE_SEPARATE_OUT_BYTES;
+  constexpr int LDS_ELEMS = SEPARATE_OUT ? FV_ELEMS + OUT_ELEMS : (FV_ELEMS > OUT_ELEMS ? FV_ELEMS : OUT_ELEMS);
+  __shared__ V s_fv[LDS_ELEMS];
+  __shared__ int s_fi[FIN * TILE];
+  V* const s_out = SEPARATE_OUT ? s_fv + FV_ELEMS : s_fv;
   __shared__ unsigned s_bits[NWORDS];
   __shared__ int s_vote[NW];
   __shared__ int s_wave_key[NW];
@@ -316,7 +332,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
 
   // 1: first-level loads.  A tile holds Z <= TILE non-zeros; lanes past Z re-read the tile's last
   // edge (one cache line, no extra traffic) instead of running into the next tile's edges.
-  typename G::Fetch f[IPT];
+  Fetch f[IPT];
   const int e_last = min(y0 + max(Z - 1, 0), last_edge);
 #pragma unroll
   for (int k = 0; k < IPT; ++k) G::fetch(p, min(y0 + tid + k * BLOCK, e_last), f[k]);
@@ -338,31 +354,16 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
     }
   }
 
-  // 2: gathers
-  typename G::Gather g[IPT];
-#pragma unroll
-  for (int k = 0; k < IPT; ++k) G::gather(p, f[k], g[k]);
-
   if (tid < NWORDS) s_bits[tid] = 0u;
 
-  // 3: map in coalesced order.  Without side effects it runs for every lane (slots past Z are never
-  // read back as non-zeros); with stores or stage-1 aggregators it is predicated.
-  Pack<V, AGG> agg;
-  zero(agg);
+  // 2: hand-over through LDS, in coalesced order.  Every slot of the tile is written (slots past Z hold
+  // copies of the tile's last edge), so a clamped read always finds a real edge.
 #pragma unroll
-  for (int k = 0; k < IPT; ++k) {
-    const int j = k * BLOCK + tid;
-    if (G::STAGE1_PURE || j < Z) {
-      Pack<V, XCH> xv;
-      G::stage1(p, y0 + j, f[k], g[k], xv, agg);
-#pragma unroll
-      for (int c = 0; c < XCH; ++c) s_xch[c * TILE + j] = xv.v[c];
-    }
-  }
+  for (int k = 0; k < IPT; ++k) G::template put<TILE>(f[k], s_fv, s_fi, k * BLOCK + tid);
 
-  // 4: vote - can every row of this tile be summed by one thread?  Row i of the tile spans the
+  // vote - can every row of this tile be summed by one thread?  Row i of the tile spans the
   // tile-relative non-zeros [end(i-1), end(i)), with end(-1) = 0 and, for the row still open at the
-  // end of the tile (i == R), end = Z.  The vote doubles as the barrier that publishes s_xch.
+  // end of the tile (i == R), end = Z.
   const bool few_rows = (R + 1 <= ROW_PATH_MAX_ROWS);
   int start1 = 0, len1 = 0, start2 = 0, len2 = 0;
   {
@@ -406,42 +407,42 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
   const bool irregular = any_vote != 0;
 #endif
 
+  Pack<V, AGG> agg;
+  zero(agg);
+
   if (!irregular) {
     // ---------------- ROW path ----------------
     auto sum_row = [&](const int r, const int start, const int len, const Pack<V, ROW>& rv) {
-      Pack<V, XCH> xv[ROW_PATH_UNROLL];
-#pragma unroll
-      for (int it = 0; it < ROW_PATH_UNROLL; ++it) {
-        const int yi = min(start + it, TILE - 1);
-#pragma unroll
-        for (int c = 0; c < XCH; ++c) xv[it].v[c] = s_xch[c * TILE + yi];
-      }
       Pack<V, RED> tot;
       zero(tot);
-      auto add_edge = [&](const int yi, const Pack<V, XCH>& x) {
+      auto add_edge = [&](const int yi, const Fetch& fe, const Gather& ge) {
         Pack<V, RED> dt;
         Pack<V, AGG> da;
-        G::contrib(p, y0 + yi, x0 + r, x, rv, dt, da);
+        G::edge(p, y0 + yi, fe, ge, rv, dt, da);
 #pragma unroll
         for (int c = 0; c < RED; ++c) tot.v[c] += dt.v[c];
 #pragma unroll
-        for (int c = 0; c < AGG; ++c)
-          if ((G::AGG2_MASK >> c) & 1u) agg.v[c] += da.v[c];
+        for (int c = 0; c < AGG; ++c) agg.v[c] += da.v[c];
       };
+      // ROW_PATH_UNROLL edges at a time: LDS reads, then all their gathers, then the arithmetic.  The
+      // first group is unconditional (lanes of shorter rows read clamped slots and discard the result).
+      for (int base = 0; base == 0 || base < len; base += ROW_PATH_UNROLL) {
+        Fetch fe[ROW_PATH_UNROLL];
+        Gather ge[ROW_PATH_UNROLL];
 #pragma unroll
-      for (int it = 0; it < ROW_PATH_UNROLL; ++it) {
-        if (it < len) {
+        for (int it = 0; it < ROW_PATH_UNROLL; ++it)
+          G::template get<TILE>(s_fv, s_fi, min(start + base + it, TILE - 1), fe[it]);
+#pragma unroll
+        for (int it = 0; it < ROW_PATH_UNROLL; ++it) G::gather(p, fe[it], ge[it]);
+#pragma unroll
+        for (int it = 0; it < ROW_PATH_UNROLL; ++it) {
+          if (base + it < len) {
 #ifdef FLEX_TUNE_ROW_BRANCH  // tuning switch: keep the predicate as a branch on the exec mask instead of selects
-          asm volatile("" ::: "memory");
+            asm volatile("" ::: "memory");
 #endif
-          add_edge(start + it, xv[it]);
+            add_edge(start + base + it, fe[it], ge[it]);
+          }
         }
-      }
-      for (int it = ROW_PATH_UNROLL; it < len; ++it) {
-        Pack<V, XCH> x;
-#pragma unroll
-        for (int c = 0; c < XCH; ++c) x.v[c] = s_xch[c * TILE + start + it];
-        add_edge(start + it, x);
       }
       if (r < R) {
         G::store_row(p, x0 + r, tot);
@@ -456,6 +457,36 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
     if (wave == 0 && BLOCK + tid <= R) sum_row(BLOCK + tid, start2, len2, rowv2);
   } else {
     // ---------------- MERGE path ----------------
+    // Graphs without row-aligned sources run the map here, in coalesced edge order, from the registers of
+    // the first-level loads (neighbouring lanes hold neighbouring edges of a row, whose columns ascend: the
+    // gathers of a power-law matrix hit the same lines far more often than in per-thread item order) and
+    // hand the contributions to the walk through LDS.  Graphs with row-aligned sources need the row of
+    // every edge first: their walk takes the fetched data from LDS and gathers per item.
+    constexpr bool MAP_FIRST = (ROW == 0);
+    constexpr bool OUT_OVERLAPS = !SEPARATE_OUT || (MAP_FIRST && RED > FVN);  // s_out over data the walk reads
+    V* const s_x = s_fv;  // MAP_FIRST: contributions [c * TILE + j]; nobody reads s_fv after the vote
+    if constexpr (MAP_FIRST) {
+      const Pack<V, ROW> no_row{};
+#pragma unroll
+      for (int k0 = 0; k0 < IPT; k0 += MERGE_CHUNK) {
+        Gather g[MERGE_CHUNK];
+#pragma unroll
+        for (int k = 0; k < MERGE_CHUNK; ++k) G::gather(p, f[k0 + k], g[k]);
+#pragma unroll
+        for (int k = 0; k < MERGE_CHUNK; ++k) {
+          const int j = (k0 + k) * BLOCK + tid;
+          if (G::EDGE_PURE || j < Z) {
+            Pack<V, RED> dt;
+            Pack<V, AGG> da;
+            G::edge(p, y0 + j, f[k0 + k], g[k], no_row, dt, da);
+#pragma unroll
+            for (int c = 0; c < RED; ++c) s_x[c * TILE + j] = dt.v[c];
+#pragma unroll
+            for (int c = 0; c < AGG; ++c) agg.v[c] += (j < Z) ? da.v[c] : V(0);
+          }
+        }
+      }
+    }
     // row ends -> bitmap over merge positions (rows beyond the prefetched ones are read here)
     if (tid < R) {
       const int pos = (re - y0) + tid;
@@ -492,58 +523,68 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
     const int xs = word_prefix + __popc(word & ((1u << sh) - 1u));                    // rows before my items
     const int ys = d0 - xs;                                                            // non-zeros before them
 
-    Pack<V, XCH> xv[IPT];
+    // what the walk needs for my items, from LDS (a row-end item reads the edge after it: harmless):
+    // the contributions (MAP_FIRST) or the fetched data
+    Pack<V, RED> xv[MAP_FIRST ? IPT : 1];
+    Fetch fe[MAP_FIRST ? 1 : IPT];
     int xrel[IPT];
 #pragma unroll
     for (int it = 0; it < IPT; ++it) {
       const int before = __popc(ends & ((1u << it) - 1u));
       xrel[it] = xs + before;
       const int yi = ys + it - before;  // < TILE by construction
+      if constexpr (MAP_FIRST) {
 #pragma unroll
-      for (int c = 0; c < XCH; ++c) xv[it].v[c] = s_xch[c * TILE + yi];
+        for (int c = 0; c < RED; ++c) xv[it].v[c] = s_x[c * TILE + yi];
+      } else {
+        G::template get<TILE>(s_fv, s_fi, yi, fe[it]);
+      }
     }
 
-    if constexpr (!SEPARATE_OUT) __syncthreads();  // every thread has read its s_xch values: the buffer now serves as s_out
+    if constexpr (OUT_OVERLAPS) __syncthreads();  // every thread has read its items: the buffer now serves as s_out
 
     Pack<V, RED> tot;
     zero(tot);
     const int dump = OUT_CAP + lane;
 #pragma unroll
-    for (int it = 0; it < IPT; ++it) {
-      const bool nz = (nzs >> it) & 1u;
-      const bool end = (ends >> it) & 1u;
-      Pack<V, RED> dt;
-      Pack<V, AGG> da;
-      Pack<V, ROW> rv;
-      if constexpr (G::STAGE2_PURE && ROW == 0) {
-        // the contribution of a non-zero is computed for every item and masked in
-        G::contrib(p, y0 + ys + it - (xrel[it] - xs), x0 + xrel[it], xv[it], rv, dt, da);
+    for (int it0 = 0; it0 < IPT; it0 += MERGE_CHUNK) {
+      Gather ge[MERGE_CHUNK];
+      if constexpr (!MAP_FIRST) {
 #pragma unroll
-        for (int c = 0; c < RED; ++c) tot.v[c] += nz ? dt.v[c] : V(0);
+        for (int k = 0; k < MERGE_CHUNK; ++k) G::gather(p, fe[it0 + k], ge[k]);
+      }
 #pragma unroll
-        for (int c = 0; c < AGG; ++c)
-          if ((G::AGG2_MASK >> c) & 1u) agg.v[c] += nz ? da.v[c] : V(0);
-      } else {
-        if (nz) {
-          // row-aligned sources are read from memory here: graphs that use them are mesh-like and
-          // take the row path, so this is the uncommon case
-          if constexpr (ROW > 0) G::load_row(p, x0 + xrel[it], rv);
-          G::contrib(p, y0 + ys + it - (xrel[it] - xs), x0 + xrel[it], xv[it], rv, dt, da);
+      for (int k = 0; k < MERGE_CHUNK; ++k) {
+        const int it = it0 + k;
+        const bool nz = (nzs >> it) & 1u;
+        const bool end = (ends >> it) & 1u;
+        if constexpr (MAP_FIRST) {
 #pragma unroll
-          for (int c = 0; c < RED; ++c) tot.v[c] += dt.v[c];
+          for (int c = 0; c < RED; ++c) tot.v[c] += nz ? xv[it].v[c] : V(0);
+        } else {
+          if (nz) {
+            // row-aligned sources are read from memory here: graphs that use them are mesh-like and
+            // take the row path, so this is the uncommon case
+            Pack<V, RED> dt;
+            Pack<V, AGG> da;
+            Pack<V, ROW> rv;
+            G::load_row(p, x0 + xrel[it], rv);
+            G::edge(p, y0 + ys + it - (xrel[it] - xs), fe[it], ge[k], rv, dt, da);
 #pragma unroll
-          for (int c = 0; c < AGG; ++c)
-            if ((G::AGG2_MASK >> c) & 1u) agg.v[c] += da.v[c];
+            for (int c = 0; c < RED; ++c) tot.v[c] += dt.v[c];
+#pragma unroll
+            for (int c = 0; c < AGG; ++c) agg.v[c] += da.v[c];
+          }
         }
-      }
-      // a row end parks the finished total in the output buffer (other items write a dump slot)
-      {
-        const int slot = end ? xrel[it] : dump;
+        // a row end parks the finished total in the output buffer (other items write a dump slot)
+        {
+          const int slot = end ? xrel[it] : dump;
 #pragma unroll
-        for (int c = 0; c < RED; ++c) s_out[c * OUT_STRIDE + slot] = tot.v[c];
-      }
+          for (int c = 0; c < RED; ++c) s_out[c * OUT_STRIDE + slot] = tot.v[c];
+        }
 #pragma unroll
-      for (int c = 0; c < RED; ++c) tot.v[c] = end ? V(0) : tot.v[c];
+        for (int c = 0; c < RED; ++c) tot.v[c] = end ? V(0) : tot.v[c];
+      }
     }
 
     // block-wide segmented scan of the open totals, keyed by the row each thread ended in
@@ -733,8 +774,11 @@ flat_kernel(const typename G::Params p, const int nnz, const int num_tiles,
     for (int k = 0; k < IPT; ++k) {
       const long long e = base + k * BLOCK + tid;
       if (e < nnz) {
-        Pack<V, G::XCH_WIDTH> unused;
-        G::stage1(p, (int)e, f[k], g[k], unused, agg);
+        Pack<V, 0> no_row, no_total;
+        Pack<V, AGG> da;
+        G::edge(p, (int)e, f[k], g[k], no_row, no_total, da);
+#pragma unroll
+        for (int c = 0; c < AGG; ++c) agg.v[c] += da.v[c];
       }
     }
   }

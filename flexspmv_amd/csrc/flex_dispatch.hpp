@@ -158,6 +158,12 @@ struct Dispatch {
         t.snap_mask = snap_rows - 1;
         t.nominal = TILE - (int)slack;
         t.xcd_shift = FLEX_TUNE_XCD_RUN_SHIFT;  // short rows: neighbouring tiles gather neighbouring data
+#ifndef FLEX_TUNE_NO_ROW_CAP
+        // a thread per row: a tile of more than BLOCK average rows sends its first wavefront through a
+        // second pass (a whole gather - map - store chain for a handful of rows)
+        const int64_t block_rows_items = (int64_t)BLOCK * (num_rows + ne) / num_rows;
+        if (block_rows_items < t.nominal && block_rows_items >= TILE / 2) t.nominal = (int)block_rows_items;
+#endif
       }
     }
     const int64_t items = REDUCER ? num_rows + ne : ne;

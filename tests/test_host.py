@@ -65,26 +65,31 @@ def test_shape_rule_and_unknown_op():
 # ---------------------------------------------------------------------------------------------
 # generator: stage split, widths, policy
 # ---------------------------------------------------------------------------------------------
-def test_stage_split_of_row_aligned_selector():
+def test_memory_levels_of_a_graph():
     kp = analyse(graphs.get("spmv_dot"))
-    assert kp.vars["mul"].stage == 1 and kp.vars["mul_1"].stage == 2 and kp.vars["selector_row"].stage == 2
-    assert (kp.xch_width, kp.red_width, kp.agg_width, kp.row_width) == (1, 1, 1, 1)
+    assert [v[0] for v in kp.fetch_values] == ["vals"] and kp.fetch_indices == [("selector_col", 0)]
+    assert [g[0] for g in kp.gathers] == ["selector_col"] and [r[0] for r in kp.row_sources] == ["selector_row"]
+    assert (kp.fetch_value_width, kp.fetch_index_width, kp.red_width, kp.agg_width, kp.row_width) == (1, 1, 1, 1, 1)
     src, sig = generate_hip_source(graphs.get("spmv_dot"))
-    assert sig["row_aligned_index_inputs"] == ["selector_row_idx"]
-    assert "p.selector_row_ptr" not in src.split("static FLEX_DEV void fetch")[1]   # never dereferenced
-    # the mesh maps would have to push every input through LDS: their row selector is read like any other
+    assert sig["row_aligned_index_inputs"] == ["selector_row_idx"] and sig["row_indexed_value_inputs"] == ["x"]
+    assert "selector_row_idx_ptr +" not in src                                   # never dereferenced
+    # the mesh maps: the destination selector comes from the row as well, the source selector is gathered
     kp = analyse(graphs.get("spring_mass"))
-    assert kp.row_width == 0 and kp.red_width == 3 and kp.agg_width == 1 and kp.xch_width == 3
+    assert (kp.fetch_value_width, kp.fetch_index_width, kp.red_width, kp.agg_width, kp.row_width) == (2, 1, 3, 1, 3)
     _, sig = generate_hip_source(graphs.get("spring_mass"))
-    assert sig["row_aligned_index_inputs"] == []
+    assert sig["row_aligned_index_inputs"] == ["gather_dst_idx"] and sig["row_indexed_value_inputs"] == ["pos"]
+    kp = analyse(graphs.get("swe_rusanov"))
+    assert (kp.fetch_value_width, kp.fetch_index_width, kp.red_width, kp.row_width) == (3, 1, 3, 3)
 
 
-def test_plain_spmv_exchanges_only_its_products():
+def test_plain_spmv_hands_over_value_and_column():
     kp = analyse(graphs.get("csr_spmv"))
-    assert (kp.xch_width, kp.row_width, kp.agg_width) == (1, 0, 0)
+    assert (kp.fetch_value_width, kp.fetch_index_width, kp.row_width, kp.agg_width) == (1, 1, 0, 0)
     src, sig = generate_hip_source(graphs.get("csr_spmv"))
     assert sig["policy"]["block"] == 256 and sig["policy"]["ipt"]["float64"] == 8
-    assert "STAGE1_PURE = true" in src and "STAGE2_PURE = true" in src
+    assert "EDGE_PURE = true" in src
+    src, _ = generate_hip_source(graphs.get("map_store"))
+    assert "EDGE_PURE = false" in src                                            # it stores per edge
 
 
 def test_policy_shrinks_tile_for_wide_graphs():
