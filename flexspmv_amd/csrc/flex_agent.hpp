@@ -113,6 +113,7 @@ struct Tiling {
   int snap_slack;  // 0: boundaries stay on their diagonals
   int snap_mask;   // rows per output line - 1 (power of two - 1)
   int xcd_shift;   // runs of 2^xcd_shift consecutive tiles share an XCD (see tile_of_block)
+  int row_group;   // row path: edges of a row staged at a time (<= the kernel's register budget; 0: that budget)
 };
 
 __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end, int num_rows,
@@ -132,18 +133,25 @@ __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int
   return c;
 }
 
-// The same boundary found by a whole wavefront (all 64 lanes must call it; the result is uniform).
-// A search by one lane is a chain of dependent loads; here a round is one load per lane.  Up to three
-// rounds probe 64 consecutive rows around a guess: first the interpolated position, then that position
-// corrected by the residual at the edge of the window just probed (a Newton step with a 64-row
-// window).  Regular matrices end after one round, smoothly varying ones after two.  If that fails the
-// bracket shrinks 64-fold per round.  The row-start load of a snapped boundary is served from the
-// probes of the round that found the answer when that row is among them.  Result: identical to
-// tile_boundary (same monotone predicate, same rule).
-__device__ __forceinline__ int2 wave_tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end,
-                                                   int num_rows, int nnz) {
-  constexpr int LEAD = 40;  // rows of the window below the guess (covers the row a snap moves back to)
+// The same boundary found by a group of W consecutive lanes (W = 8, 16, 32 or 64; all lanes of the group
+// must call it; the result is the same in every lane of the group).  A search by one lane is a chain of
+// dependent loads; here a link of the chain is one load per lane.  Up to three rounds probe W consecutive
+// rows around a guess: first the interpolated position, then that position corrected by the residual at
+// the edge of the window just probed (a Newton step with a W-row window).  Regular matrices end after
+// one or two rounds.  If that fails the bracket shrinks W-fold per round.  The row-start load of a
+// snapped boundary is served from the probes of the round that found the answer when that row is among
+// them.  Result: identical to tile_boundary (same monotone predicate, same rule).
+template <int W>
+__device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end,
+                                                    int num_rows, int nnz) {
+  static_assert(W == 8 || W == 16 || W == 32 || W == 64, "group width");
+  constexpr int LEAD = (W * 5) / 8;  // rows of the window below the guess (towards the row a snap moves back to)
   const int lane = lane_id();
+  const int gbase = lane & ~(W - 1);  // first lane of my group
+  const int glane = lane & (W - 1);
+  constexpr unsigned long long GMASK = (W == 64) ? ~0ull : ((1ull << (W & 63)) - 1ull);
+  auto group_ballot = [&](bool b) { return (__builtin_amdgcn_ballot_w64(b) >> gbase) & GMASK; };
+  auto from_lane = [&](int v, int l) { return __builtin_amdgcn_ds_bpermute((gbase + l) << 2, v); };
   const long long d = (long long)t * tl.nominal;
   const int diag = (int)min(d, (long long)num_rows + nnz);
   int lo = max(diag - nnz, 0);
@@ -155,18 +163,18 @@ __device__ __forceinline__ int2 wave_tile_boundary(int t, const Tiling& tl, cons
   bool win_valid = false;
 #pragma unroll 1
   for (int round = 0; round < 3 && lo < hi; ++round) {
-    const int w0 = min(max(guess - LEAD, lo), max(hi - WAVE, lo));  // window [w0, w0 + 64) inside [lo, hi)
-    const int pos = w0 + lane;
+    const int w0 = min(max(guess - LEAD, lo), max(hi - W, lo));  // window [w0, w0 + W) inside [lo, hi)
+    const int pos = w0 + glane;
     int end = 0;
     bool past = true;  // lanes at or beyond hi behave like "predicate true"
     if (pos < hi) {
       end = row_end[pos];
       past = end + pos + 1 > diag;
     }
-    const unsigned long long m = __builtin_amdgcn_ballot_w64(past);
+    const unsigned long long m = group_ballot(past);
     if (m == 0ull) {  // every probed row ends before the diagonal: the answer lies beyond the window
-      const int g_last = __builtin_amdgcn_readlane(end, WAVE - 1) + (w0 + WAVE - 1) + 1;
-      lo = w0 + WAVE;
+      const int g_last = from_lane(end, W - 1) + (w0 + W - 1) + 1;
+      lo = w0 + W;
       guess = (int)min((long long)lo + (long long)((float)(diag - g_last) * inv_slope), (long long)hi);
     } else {
       const int j = __builtin_ctzll(m);
@@ -176,39 +184,36 @@ __device__ __forceinline__ int2 wave_tile_boundary(int t, const Tiling& tl, cons
         win_end_value = end;
         win_valid = true;
       } else {  // the answer is at or before the window's first row
-        const int g_first = __builtin_amdgcn_readlane(end, 0) + w0 + 1;
+        const int g_first = from_lane(end, 0) + w0 + 1;
         hi = w0;
         guess = w0 - 1 - (int)((float)(g_first - diag) * inv_slope);
       }
     }
-    lo = __builtin_amdgcn_readfirstlane(lo);  // uniform by construction; tell the compiler
-    hi = __builtin_amdgcn_readfirstlane(hi);
-    guess = __builtin_amdgcn_readfirstlane(guess);
   }
   const int probed_below = min(diag, num_rows);  // window lanes at or beyond this row hold no probe
 #pragma unroll 1
-  while (lo < hi) {  // 64 evenly spaced probes per round
+  while (lo < hi) {  // W evenly spaced probes per round
     const int n = hi - lo;
-    const int step = (n + WAVE - 1) / WAVE;
-    const int pos = lo + (lane + 1) * step - 1;
+    const int step = (n + W - 1) / W;
+    const int pos = lo + (glane + 1) * step - 1;
     bool past = true;
     if (pos < hi) past = row_end[pos] + pos + 1 > diag;
-    const unsigned long long m = __builtin_amdgcn_ballot_w64(past);
-    const int j = (m == 0ull) ? WAVE : __builtin_ctzll(m);
+    const unsigned long long m = group_ballot(past);
+    const int j = (m == 0ull) ? W : __builtin_ctzll(m);
     // samples before j end before the diagonal, sample j (if any) does not
-    const int new_lo = min(lo + j * step, hi);                                    // one past sample j - 1
-    const int new_hi = (j == WAVE) ? hi : min(lo + (j + 1) * step - 1, hi);      // sample j itself (or hi)
-    lo = __builtin_amdgcn_readfirstlane(new_lo);
-    hi = __builtin_amdgcn_readfirstlane(new_hi);
+    const int new_lo = min(lo + j * step, hi);                               // one past sample j - 1
+    const int new_hi = (j == W) ? hi : min(lo + (j + 1) * step - 1, hi);    // sample j itself (or hi)
+    lo = new_lo;
+    hi = new_hi;
   }
   int2 c = make_int2(min(lo, num_rows), diag - lo);
   if (tl.snap_slack > 0 && t > 0 && t < tl.num_tiles) {
     const int xs = c.x & ~tl.snap_mask;
     int ys = 0;
     if (xs > 0) {
-      const int src = xs - 1 - win_start;  // lane that probed row xs - 1
-      if (win_valid && src >= 0 && src < WAVE && xs - 1 < probed_below) {
-        ys = __builtin_amdgcn_readfirstlane(__builtin_amdgcn_ds_bpermute(src << 2, win_end_value));
+      const int src = xs - 1 - win_start;  // lane of the group that probed row xs - 1
+      if (win_valid && src >= 0 && src < W && xs - 1 < probed_below) {
+        ys = from_lane(win_end_value, src);
       } else {
         ys = row_end[xs - 1];
       }
@@ -218,12 +223,33 @@ __device__ __forceinline__ int2 wave_tile_boundary(int t, const Tiling& tl, cons
   return c;
 }
 
+// ... by a whole wavefront: the result is uniform, which the compiler is told
+__device__ __forceinline__ int2 wave_tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end,
+                                                   int num_rows, int nnz) {
+  int2 c = group_tile_boundary<WAVE>(t, tl, row_end, num_rows, nnz);
+  c.x = __builtin_amdgcn_readfirstlane(c.x);
+  c.y = __builtin_amdgcn_readfirstlane(c.y);
+  return c;
+}
+
 // One search per tile boundary: coords[t] is where tile t starts, coords[num_tiles] where the path ends.
-__global__ void __launch_bounds__(256)
+// SEARCH_GROUP lanes per boundary: enough to cut the chain of dependent loads to two or three links, few
+// enough for all boundaries of a large launch to be searched at once.
+constexpr int SEARCH_BLOCK = 256;
+#ifndef FLEX_TUNE_SEARCH_GROUP
+#define FLEX_TUNE_SEARCH_GROUP 8
+#endif
+constexpr int SEARCH_GROUP = FLEX_TUNE_SEARCH_GROUP;
+__global__ void __launch_bounds__(SEARCH_BLOCK)
 tile_search_kernel(const Tiling tl, const int* __restrict__ row_end, int num_rows, int nnz, int2* __restrict__ coords) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t > tl.num_tiles) return;
-  coords[t] = tile_boundary(t, tl, row_end, num_rows, nnz);
+  const int t = (int)(blockIdx.x * (SEARCH_BLOCK / SEARCH_GROUP) + threadIdx.x / SEARCH_GROUP);
+  if (t > tl.num_tiles) return;  // uniform per group
+#ifdef FLEX_TUNE_THREAD_SEARCH  // tuning switch: one lane searches
+  if ((threadIdx.x & (SEARCH_GROUP - 1)) == 0) coords[t] = tile_boundary(t, tl, row_end, num_rows, nnz);
+#else
+  const int2 c = group_tile_boundary<SEARCH_GROUP>(t, tl, row_end, num_rows, nnz);
+  if ((threadIdx.x & (SEARCH_GROUP - 1)) == 0) coords[t] = c;
+#endif
 }
 
 // Which tile a block works on.  Blocks are dealt to the 8 XCDs round-robin (block % 8), each XCD with
@@ -271,8 +297,8 @@ inline int grid_for_tiles(int num_tiles, int xcd_shift) {
 // ----------------------------------------------------------------------------------------------
 template <class G, int BLOCK, int IPT>
 __device__ __forceinline__ void
-reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, const int* __restrict__ row_end,
-            const int nnz, const typename G::Params& p, int* __restrict__ carry_row,
+reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hint, const int num_rows,
+            const int* __restrict__ row_end, const int nnz, const typename G::Params& p, int* __restrict__ carry_row,
             typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials) {
   using V = typename G::Value;
   using Fetch = typename G::Fetch;
@@ -412,6 +438,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
 
   if (!irregular) {
     // ---------------- ROW path ----------------
+    const int group = (row_group_hint > 0 && row_group_hint < ROW_PATH_UNROLL) ? row_group_hint : ROW_PATH_UNROLL;
     auto sum_row = [&](const int r, const int start, const int len, const Pack<V, ROW>& rv) {
       Pack<V, RED> tot;
       zero(tot);
@@ -424,19 +451,23 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int num_rows, co
 #pragma unroll
         for (int c = 0; c < AGG; ++c) agg.v[c] += da.v[c];
       };
-      // ROW_PATH_UNROLL edges at a time: LDS reads, then all their gathers, then the arithmetic.  The
-      // first group is unconditional (lanes of shorter rows read clamped slots and discard the result).
-      for (int base = 0; base == 0 || base < len; base += ROW_PATH_UNROLL) {
+      // A group of edges at a time: LDS reads, then all their gathers, then the arithmetic.  The group is
+      // as large as the register budget allows, cut down to the launch's average row length (a slot no
+      // row uses still costs every lane a gather); the cut is the same for all lanes, so it is a scalar
+      // branch.  The first group is unconditional (lanes of shorter rows read clamped slots and
+      // discard the result).
+      for (int base = 0; base == 0 || base < len; base += group) {
         Fetch fe[ROW_PATH_UNROLL];
         Gather ge[ROW_PATH_UNROLL];
 #pragma unroll
         for (int it = 0; it < ROW_PATH_UNROLL; ++it)
-          G::template get<TILE>(s_fv, s_fi, min(start + base + it, TILE - 1), fe[it]);
+          if (it < group) G::template get<TILE>(s_fv, s_fi, min(start + base + it, TILE - 1), fe[it]);
 #pragma unroll
-        for (int it = 0; it < ROW_PATH_UNROLL; ++it) G::gather(p, fe[it], ge[it]);
+        for (int it = 0; it < ROW_PATH_UNROLL; ++it)
+          if (it < group) G::gather(p, fe[it], ge[it]);
 #pragma unroll
         for (int it = 0; it < ROW_PATH_UNROLL; ++it) {
-          if (base + it < len) {
+          if (it < group && base + it < len) {
 #ifdef FLEX_TUNE_ROW_BRANCH  // tuning switch: keep the predicate as a branch on the exec mask instead of selects
             asm volatile("" ::: "memory");
 #endif
@@ -696,7 +727,7 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
       n0 = coords[next];
       n1 = coords[next + 1];
     }
-    reduce_tile<G, BLOCK, IPT>(tile, c0, c1, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
+    reduce_tile<G, BLOCK, IPT>(tile, c0, c1, tl.row_group, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
     if (!more) break;
     __syncthreads();  // the tile's LDS is free again
     tile = next;
@@ -740,7 +771,7 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
       if (tile == num_tiles - 1) coords_out[num_tiles] = c1;
     }
   }
-  reduce_tile<G, BLOCK, IPT>(tile, c0, c1, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
+  reduce_tile<G, BLOCK, IPT>(tile, c0, c1, tl.row_group, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
 #endif
 }
 

@@ -150,6 +150,7 @@ struct Dispatch {
     t.snap_slack = 0;
     t.snap_mask = 0;
     t.xcd_shift = 0;
+    t.row_group = 0;
     if (REDUCER && FLEX_TUNE_SNAP_BYTES > 0 && num_rows > 0) {
       const int snap_rows = FLEX_TUNE_SNAP_BYTES / (int)sizeof(V) > 1 ? FLEX_TUNE_SNAP_BYTES / (int)sizeof(V) : 1;
       const int64_t slack = (snap_rows * (num_rows + ne) + num_rows - 1) / num_rows;  // snap_rows average rows
@@ -158,6 +159,9 @@ struct Dispatch {
         t.snap_mask = snap_rows - 1;
         t.nominal = TILE - (int)slack;
         t.xcd_shift = FLEX_TUNE_XCD_RUN_SHIFT;  // short rows: neighbouring tiles gather neighbouring data
+#ifndef FLEX_TUNE_NO_ROW_GROUP
+        t.row_group = (int)((ne + num_rows - 1) / num_rows);  // average row length, rounded up
+#endif
 #ifndef FLEX_TUNE_NO_ROW_CAP
         // a thread per row: a tile of more than BLOCK average rows sends its first wavefront through a
         // second pass (a whole gather - map - store chain for a handful of rows)
@@ -273,9 +277,10 @@ struct Dispatch {
       V* carry_val = (V*)(ws + l.off_carry_val);
 
       if (!l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0) {
-        const int search_blocks = (l.num_tiles + 1 + 255) / 256;
-        hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(256), 0, stream, l.tiling, row_end, num_rows,
-                           nnz, coords);
+        constexpr int per_block = SEARCH_BLOCK / SEARCH_GROUP;
+        const int search_blocks = (l.num_tiles + 1 + per_block - 1) / per_block;
+        hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(SEARCH_BLOCK), 0, stream, l.tiling, row_end,
+                           num_rows, nnz, coords);
       }
       if (timed) (void)hipEventRecord(g_timer.start, stream);
 #ifdef FLEX_TUNE_PERSISTENT
