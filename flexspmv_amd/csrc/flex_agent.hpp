@@ -31,6 +31,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "flex_tensor.hpp"
 #include "flex_wave.hpp"
 
@@ -327,7 +329,9 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   constexpr int MERGE_CHUNK = ROW_PATH_UNROLL < IPT ? ROW_PATH_UNROLL : IPT;  // likewise in the merge walk
   constexpr int ROW_PATH_MAX_ROWS = BLOCK + WAVE;  // rows (incl. the open one) whose ends are prefetched
   static_assert((IPT & (IPT - 1)) == 0 && IPT <= 32, "a thread's items must sit inside one bitmap word");
+#ifndef FLEX_TUNE_UNSAFE_BIG_TILE  // experiment switch: row path only (the merge path would be wrong)
   static_assert(NWORDS <= WAVE, "one wavefront scans the bitmap words");
+#endif
 
   // s_fv / s_fi hold what was fetched for the tile's edges, s_out the rows the merge path finishes.
   // Where both fit a modest budget they are separate; otherwise s_out reuses s_fv after a barrier.
@@ -438,54 +442,61 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
 
   if (!irregular) {
     // ---------------- ROW path ----------------
-    const int group = (row_group_hint > 0 && row_group_hint < ROW_PATH_UNROLL) ? row_group_hint : ROW_PATH_UNROLL;
-    auto sum_row = [&](const int r, const int start, const int len, const Pack<V, ROW>& rv) {
-      Pack<V, RED> tot;
-      zero(tot);
-      auto add_edge = [&](const int yi, const Fetch& fe, const Gather& ge) {
-        Pack<V, RED> dt;
-        Pack<V, AGG> da;
-        G::edge(p, y0 + yi, fe, ge, rv, dt, da);
+    // A row's edges are handled a group at a time: LDS reads, then all their gathers, then the arithmetic.
+    // The group is as large as the register budget allows, cut down to the launch's average row length
+    // (a slot no row uses still costs every lane a gather).  The first group is unconditional (lanes of
+    // shorter rows read clamped slots and discard the result).  The group size is a compile-time constant
+    // of the code that runs: one copy of the row path per size between the budget and half of it.
+    auto row_path = [&](auto group_tag) {
+      constexpr int GROUP = decltype(group_tag)::value;
+      auto sum_row = [&](const int r, const int start, const int len, const Pack<V, ROW>& rv) {
+        Pack<V, RED> tot;
+        zero(tot);
+        auto add_edge = [&](const int yi, const Fetch& fe, const Gather& ge) {
+          Pack<V, RED> dt;
+          Pack<V, AGG> da;
+          G::edge(p, y0 + yi, fe, ge, rv, dt, da);
 #pragma unroll
-        for (int c = 0; c < RED; ++c) tot.v[c] += dt.v[c];
+          for (int c = 0; c < RED; ++c) tot.v[c] += dt.v[c];
 #pragma unroll
-        for (int c = 0; c < AGG; ++c) agg.v[c] += da.v[c];
-      };
-      // A group of edges at a time: LDS reads, then all their gathers, then the arithmetic.  The group is
-      // as large as the register budget allows, cut down to the launch's average row length (a slot no
-      // row uses still costs every lane a gather); the cut is the same for all lanes, so it is a scalar
-      // branch.  The first group is unconditional (lanes of shorter rows read clamped slots and
-      // discard the result).
-      for (int base = 0; base == 0 || base < len; base += group) {
-        Fetch fe[ROW_PATH_UNROLL];
-        Gather ge[ROW_PATH_UNROLL];
+          for (int c = 0; c < AGG; ++c) agg.v[c] += da.v[c];
+        };
+        for (int base = 0; base == 0 || base < len; base += GROUP) {
+          Fetch fe[GROUP];
+          Gather ge[GROUP];
 #pragma unroll
-        for (int it = 0; it < ROW_PATH_UNROLL; ++it)
-          if (it < group) G::template get<TILE>(s_fv, s_fi, min(start + base + it, TILE - 1), fe[it]);
+          for (int it = 0; it < GROUP; ++it) G::template get<TILE>(s_fv, s_fi, min(start + base + it, TILE - 1), fe[it]);
 #pragma unroll
-        for (int it = 0; it < ROW_PATH_UNROLL; ++it)
-          if (it < group) G::gather(p, fe[it], ge[it]);
+          for (int it = 0; it < GROUP; ++it) G::gather(p, fe[it], ge[it]);
 #pragma unroll
-        for (int it = 0; it < ROW_PATH_UNROLL; ++it) {
-          if (it < group && base + it < len) {
+          for (int it = 0; it < GROUP; ++it) {
+            if (base + it < len) {
 #ifdef FLEX_TUNE_ROW_BRANCH  // tuning switch: keep the predicate as a branch on the exec mask instead of selects
-            asm volatile("" ::: "memory");
+              asm volatile("" ::: "memory");
 #endif
-            add_edge(start + base + it, fe[it], ge[it]);
+              add_edge(start + base + it, fe[it], ge[it]);
+            }
           }
         }
-      }
-      if (r < R) {
-        G::store_row(p, x0 + r, tot);
-      } else {  // r == R: the row still open at the end of the tile becomes the tile's carry
-        const int row = x0 + r;
-        carry_row[tile] = (row < num_rows && len > 0) ? row : -1;
+        if (r < R) {
+          G::store_row(p, x0 + r, tot);
+        } else {  // r == R: the row still open at the end of the tile becomes the tile's carry
+          const int row = x0 + r;
+          carry_row[tile] = (row < num_rows && len > 0) ? row : -1;
 #pragma unroll
-        for (int c = 0; c < RED; ++c) carry_val[(size_t)tile * RED + c] = tot.v[c];
-      }
+          for (int c = 0; c < RED; ++c) carry_val[(size_t)tile * RED + c] = tot.v[c];
+        }
+      };
+      if (tid <= R) sum_row(tid, start1, len1, rowv);
+      if (wave == 0 && BLOCK + tid <= R) sum_row(BLOCK + tid, start2, len2, rowv2);
     };
-    if (tid <= R) sum_row(tid, start1, len1, rowv);
-    if (wave == 0 && BLOCK + tid <= R) sum_row(BLOCK + tid, start2, len2, rowv2);
+    constexpr int U = ROW_PATH_UNROLL;
+    const int group = (row_group_hint > 0 && row_group_hint < U) ? row_group_hint : U;  // uniform over the launch
+    if (group >= U) row_path(std::integral_constant<int, U>{});
+    else if (U - 1 >= 2 && group == U - 1) row_path(std::integral_constant<int, (U - 1 >= 2 ? U - 1 : 2)>{});
+    else if (U - 2 >= 2 && group == U - 2) row_path(std::integral_constant<int, (U - 2 >= 2 ? U - 2 : 2)>{});
+    else if (U - 3 >= 2 && group == U - 3) row_path(std::integral_constant<int, (U - 3 >= 2 ? U - 3 : 2)>{});
+    else row_path(std::integral_constant<int, (U - 4 >= 2 ? U - 4 : 2)>{});
   } else {
     // ---------------- MERGE path ----------------
     // Graphs without row-aligned sources run the map here, in coalesced edge order, from the registers of
