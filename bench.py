@@ -303,7 +303,17 @@ def time_edge_list_preparation(w, steps):
     dst = torch.empty_like(vals)
     ms = timed(lambda: formats.gather_rows(vals, perm, out=dst), max(1, steps // 5))
     b = ne * (4 + 2 * vals.element_size() * (vals.numel() // ne))
-    out["gather_rows"] = {"ms": ms, "algorithmic_bytes": b, "gbs": b / ms / 1e6, "order": "random permutation"}
+    line_traffic = ne * (4 + 128 + vals.element_size() * (vals.numel() // ne))   # a whole 128-byte line per random read
+    out["gather_rows"] = {"ms": ms, "algorithmic_bytes": b, "gbs": b / ms / 1e6, "order": "random permutation",
+                          "line_traffic_bytes": line_traffic, "line_traffic_gbs": line_traffic / ms / 1e6}
+    # a permutation with locality: the edge list in column order (the transpose's row order)
+    cols = next((torch.from_numpy(v).cuda() for k, v in w.tensors.items()
+                 if k.endswith("_idx") and v.shape[0] == ne and not k.startswith("selector_row")), None)
+    if cols is not None:
+        _, perm_t = formats.sort_edges_by_row(cols, w.num_cols)
+        ms = timed(lambda: formats.gather_rows(vals, perm_t, out=dst), max(1, steps // 5))
+        out["gather_rows_transpose_order"] = {"ms": ms, "algorithmic_bytes": b, "gbs": b / ms / 1e6,
+                                              "order": "edges sorted by column (stable)"}
     return out
 
 

@@ -119,10 +119,10 @@ inline int resident_grid(KernelT kernel, int block_threads, GridCache& cache) {
 #define FLEX_TUNE_XCD_RUN_SHIFT 4  // launches with row-snapped tiles hand runs of 2^4 tiles to one XCD
 #endif
 #ifndef FLEX_TUNE_INBLOCK_MAX_TILES
-#define FLEX_TUNE_INBLOCK_MAX_TILES 8192  // launches of at most this many tiles search inside the reducer blocks
+#define FLEX_TUNE_INBLOCK_MAX_TILES 4096  // launches of at most this many tiles search inside the reducer blocks
 #endif
 #ifndef FLEX_TUNE_SINGLE_FIXUP_MAX_TILES
-#define FLEX_TUNE_SINGLE_FIXUP_MAX_TILES 8192  // ... and fold carries and aggregators in one block
+#define FLEX_TUNE_SINGLE_FIXUP_MAX_TILES 4096  // ... and fold carries and aggregators in one block
 #endif
 constexpr int SINGLE_FIXUP_BLOCK = 1024;
 

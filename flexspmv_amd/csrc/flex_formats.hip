@@ -165,16 +165,20 @@ hipError_t sort_pairs(void* temp, size_t& temp_bytes, const I* rows, int32_t* so
                                    permutation, (size_t)ne, 0u, (unsigned)bits_for(num_rows), stream);
 }
 
-template <bool SCATTER>
+// dst[k] = src[perm[k]] (gather) or dst[perm[k]] = src[k] (scatter) for rows of `vecs` vectors of type T.
+// One thread moves one vector; T is the widest of 16, 8 and 4 bytes that divides the row and both base
+// addresses, so an 8-byte value per edge is one load and one store (the side that follows the permutation
+// touches a cache line per row whatever the width: that line, not the instruction count, is the cost).
+template <bool SCATTER, typename T>
 __global__ void __launch_bounds__(BLOCK)
-permute_rows_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, const int32_t* __restrict__ perm,
-                    const long long n, const int words) {
+permute_rows_kernel(const T* __restrict__ src, T* __restrict__ dst, const int32_t* __restrict__ perm,
+                    const long long n, const int vecs) {
   const long long idx = (long long)blockIdx.x * BLOCK + threadIdx.x;
-  if (idx >= n * words) return;
-  const long long k = idx / words;
-  const int w = (int)(idx - k * words);
+  if (idx >= n * vecs) return;
+  const long long k = idx / vecs;
+  const int w = (int)(idx - k * vecs);
   const long long other = perm[k];
-  if (SCATTER) dst[other * words + w] = src[idx]; else dst[idx] = src[other * words + w];
+  if (SCATTER) dst[other * vecs + w] = src[idx]; else dst[idx] = src[other * vecs + w];
 }
 
 template <bool SCATTER>
@@ -184,12 +188,22 @@ int permute_rows(const void* src, void* dst, const int32_t* perm, int64_t n, int
   if (n == 0) return FLEXSPMV_FORMATS_OK;
   if (src == nullptr || dst == nullptr || perm == nullptr)
     return fail(FLEXSPMV_FORMATS_ERR_BAD_ARGUMENT, "a pointer is NULL");
-  const int64_t words = row_bytes / 4;
-  const int64_t total = n * words;
-  if (n >= ((int64_t)1 << 31) || words >= ((int64_t)1 << 20) || (total + BLOCK - 1) / BLOCK >= ((int64_t)1 << 31))
+  const uintptr_t bits = (uintptr_t)src | (uintptr_t)dst | (uintptr_t)row_bytes;
+  const int vec_bytes = (bits & 15u) == 0 ? 16 : ((bits & 7u) == 0 ? 8 : 4);
+  const int64_t vecs = row_bytes / vec_bytes;
+  const int64_t total = n * vecs;
+  if (n >= ((int64_t)1 << 31) || vecs >= ((int64_t)1 << 20) || (total + BLOCK - 1) / BLOCK >= ((int64_t)1 << 31))
     return fail(FLEXSPMV_FORMATS_ERR_TOO_LARGE, "tensor too large for one launch");
-  hipLaunchKernelGGL((permute_rows_kernel<SCATTER>), dim3((unsigned)((total + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0,
-                     (hipStream_t)stream, (const uint32_t*)src, (uint32_t*)dst, perm, (long long)n, (int)words);
+  const dim3 grid((unsigned)((total + BLOCK - 1) / BLOCK));
+  if (vec_bytes == 16)
+    hipLaunchKernelGGL((permute_rows_kernel<SCATTER, uint4>), grid, dim3(BLOCK), 0, (hipStream_t)stream,
+                       (const uint4*)src, (uint4*)dst, perm, (long long)n, (int)vecs);
+  else if (vec_bytes == 8)
+    hipLaunchKernelGGL((permute_rows_kernel<SCATTER, uint2>), grid, dim3(BLOCK), 0, (hipStream_t)stream,
+                       (const uint2*)src, (uint2*)dst, perm, (long long)n, (int)vecs);
+  else
+    hipLaunchKernelGGL((permute_rows_kernel<SCATTER, uint32_t>), grid, dim3(BLOCK), 0, (hipStream_t)stream,
+                       (const uint32_t*)src, (uint32_t*)dst, perm, (long long)n, (int)vecs);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail_hip(e, "kernel launch failed");
   return FLEXSPMV_FORMATS_OK;

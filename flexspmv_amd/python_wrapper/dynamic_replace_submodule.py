@@ -169,6 +169,10 @@ class _DynamicCudaWrapper(nn.Module):
         self._output_shapes = list(output_shapes) if output_shapes is not None else None
         self._written_inputs = set(written_inputs)
         self._dummy_ro: Dict[torch.device, torch.Tensor] = {}
+        # streamed edge tensors in the kernel's edge order, kept from the previous call: a tensor that has not
+        # changed since (same storage, same version counter - a model parameter, a mesh constant) is not
+        # permuted again
+        self._sorted_inputs: Dict[str, Tuple] = {}
 
     def _on(self, name: str, device) -> torch.Tensor:
         t = getattr(self, name)
@@ -176,6 +180,20 @@ class _DynamicCudaWrapper(nn.Module):
             t = t.to(device)
             setattr(self, name, t)
         return t
+
+    def _in_edge_order(self, name: str, t: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
+        """``t`` permuted into the kernel's edge order; the copy of the previous call when ``t`` is unchanged."""
+        if name in self._written_inputs:          # the kernel stores into the copy: always a fresh one
+            return gather_edges(t, perm)
+        storage = t.untyped_storage()
+        key = (storage.data_ptr(), t.storage_offset(), t._version, tuple(t.shape), t.dtype)
+        kept = self._sorted_inputs.get(name)
+        if kept is not None and kept[0] == key:
+            return kept[2]
+        out = gather_edges(t, perm)
+        # the storage is held so that its address cannot be handed to another tensor while the key is kept
+        self._sorted_inputs[name] = (key, storage, out)
+        return out
 
     def __call__(self, *args):
         if len(args) != len(self._input_param_names):
@@ -207,7 +225,7 @@ class _DynamicCudaWrapper(nn.Module):
                 perm = perm.to(torch.int32)
                 self.edge_permutation = perm
             for n in self._non_gather_value_inputs:
-                arg_map[n] = gather_edges(arg_map[n], perm)
+                arg_map[n] = self._in_edge_order(n, arg_map[n], perm)
         call_args = [arg_map[n] for n in self._non_gather_value_inputs]
         call_args += [arg_map[n] for n in self._gather_value_inputs]
         call_args += [self._on(b, device) for b in self._selector_buf_names]

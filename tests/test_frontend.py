@@ -337,6 +337,23 @@ def test_unsorted_reducer_rows_are_sorted_behind_the_wrapper():
     assert len(exts) >= 3
     assert torch.allclose(eager.per_row, traced.per_row, rtol=1e-13, atol=0)
     assert torch.allclose(eager.total, traced.total, rtol=1e-13, atol=0)
+    # A streamed tensor that has not changed since the previous call is not permuted again; one that was
+    # modified in place (its version counter moved) is.
+    wrappers = [m for m in compiled.modules() if type(m).__name__ == "_DynamicCudaWrapper" and m._sorted_inputs]
+    assert wrappers
+    kept = {id(w): {n: v[2] for n, v in w._sorted_inputs.items()} for w in wrappers}
+    eager()
+    compiled()
+    constant = [n for w in wrappers for n, v in w._sorted_inputs.items() if v[2] is kept[id(w)][n]]
+    assert constant                                                            # e.g. the model tensor w
+    assert torch.allclose(eager.per_row, traced.per_row, rtol=1e-13, atol=0)
+    with torch.no_grad():
+        eager.w.mul_(1.5)
+        traced.w.mul_(1.5)
+    eager()
+    compiled()
+    assert torch.equal(eager.per_edge, traced.per_edge)
+    assert torch.allclose(eager.per_row, traced.per_row, rtol=1e-13, atol=0)
 
 
 def _random_model_source(rng, n_stmts=14, rich=False):
