@@ -166,9 +166,15 @@ def time_workload(w, steps, warmup):
     return result, [o.cpu().numpy() for o in outs]
 
 
+FLOOR_ULPS = 8
+
+
 def reducer_row_scales(ir, w, run_oracle, threads):
-    """Per reducer output, the sum over each row of |what one edge contributes| (float64): the oracle run on
-    the same edges with every edge as a row of its own (single-term sums, no rounding)."""
+    """Per reducer output: (the sum over each row of |what one edge contributes| in float64, the absolute floor
+    FLOOR_ULPS * eps * largest |contribution|): the oracle run on the same edges with every edge as a row of
+    its own (single-term sums, no rounding).  The floor is what two evaluations of a map with a cancellation
+    inside (the spring's r - L) differ by however small the contribution comes out; for products it is far
+    below the row criterion."""
     import numpy as np
     ne = int(w.ne)
     per_edge, _ = run_oracle(ir, w.tensors, np.arange(ne + 1, dtype=np.int32), ne, w.num_cols, threads)
@@ -179,10 +185,11 @@ def reducer_row_scales(ir, w, run_oracle, threads):
         if spec["target"] != "reducer":
             continue
         a = np.abs(per_edge[i].astype(np.float64)).reshape(ne, -1)
+        floor = FLOOR_ULPS * float(np.finfo(per_edge[i].dtype).eps) * float(a.max())
         a = np.vstack([a, np.zeros((1, a.shape[1]))])
         s = np.add.reduceat(a, np.minimum(starts, ne), axis=0)
         s[empty] = 0.0
-        scales[i] = s
+        scales[i] = (s, floor)
     return scales
 
 
@@ -230,16 +237,17 @@ def cpu_leg(w, result, outs, cpu_runs):
         else:
             r64 = r.astype(np.float64)
         if i in scales:
-            scale = np.maximum(np.abs(r64), scales[i].reshape(r64.shape))
-            scale[scale == 0.0] = 1e-300
+            row_scale, floor = scales[i]
+            # |diff| <= tol * scale + floor  <=>  |diff| / (scale + floor / tol) <= tol
+            scale = np.maximum(np.abs(r64), row_scale.reshape(r64.shape)) + max(floor / tol, 1e-300)
             worst = max(worst, float((np.abs(o64 - r64) / scale).max()))
         else:
             worst = max(worst, float(np.abs(o64 - r64).max()) / max(float(np.abs(r64).max()), 1e-300))
     result["cpu"] = {"ms": cpu_ms, "gbs": w.algorithmic_bytes / cpu_ms / 1e6, "threads": T, "runs": cpu_runs,
                      "max_rel_diff_vs_gpu": worst, "tolerance": tol,
                      "parity_ok": bool(worst <= tol) and weak_ok, "parity_centre": centre,
-                     "parity_scale": "per row: max(|reference|, sum of |contributions| of the row); "
-                                     "aggregators: |reference|"}
+                     "parity_scale": "per row: max(|reference|, sum of |contributions| of the row) + "
+                                     f"{FLOOR_ULPS} ulp of the largest contribution / tolerance; aggregators: |reference|"}
     return result
 
 
