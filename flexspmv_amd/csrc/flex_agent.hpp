@@ -844,12 +844,18 @@ flat_kernel(const typename G::Params p, const int nnz, const int num_tiles,
 
 // ----------------------------------------------------------------------------------------------
 // Fix-up: fold tile carries into their rows (tile order) and reduce the aggregator partials.
-// A thread owns the carry of one tile at a time and, when that tile is the first of a run that carries
-// into the same row, adds the whole run to that row.  The aggregator partials (PARTS_PER_TILE per tile,
-// one per wavefront of the reducer block) are summed in a fixed order.
-//   SINGLE = false: block b handles tiles [b*BLOCK, (b+1)*BLOCK) and leaves its sum in block_partials[b];
-//                   aggregate_kernel adds those, again in a fixed order.
-//   SINGLE = true:  one block walks all tiles (launches of a few thousand tiles) and assigns the
+// Tiles are handled in chunks of BLOCK, a thread per tile.  A run of tiles that carry into the same row is
+// summed by a block-wide segmented scan (wave64 DPP scan, then a fold across the wavefronts in order); the
+// thread of the run's last tile adds the total to the row.  A run that starts in the chunk and goes on
+// beyond it - a row of millions of non-zeros - is finished by the whole block: it walks the following
+// tiles BLOCK at a time for as long as they carry into that row and adds them up in a fixed order; the
+// chunks those tiles belong to see that their leading tiles continue an earlier run and leave them alone.
+// Nothing here depends on timing: the same sums in the same order on every run, no atomics.
+// The aggregator partials (PARTS_PER_TILE per tile, one per wavefront of the reducer block) are summed in a
+// fixed order.
+//   SINGLE = false: block b handles tiles [b*BLOCK, (b+1)*BLOCK) and leaves its aggregator sum in
+//                   block_partials[b]; aggregate_kernel adds those, again in a fixed order.
+//   SINGLE = true:  one block walks all chunks (launches of a few thousand tiles) and assigns the
 //                   aggregator outputs itself: one kernel less.
 // (Finishing the sum in the last fix-up block to finish, found with a ticket counter, was measured and
 // is slower: the release fence each block needs writes the XCD's whole L2 back, output rows included.)
@@ -861,42 +867,126 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
              typename G::Value* __restrict__ block_partials) {
   using V = typename G::Value;
   constexpr int RED = G::RED_WIDTH, AGG = G::AGG_WIDTH;
+  constexpr int REDN = RED > 0 ? RED : 1;
   constexpr int NW = BLOCK / WAVE;
-  const int first = SINGLE ? (int)threadIdx.x : (int)(blockIdx.x * BLOCK + threadIdx.x);
-  const int stride = SINGLE ? BLOCK : num_tiles;  // not SINGLE: one tile per thread
+  const int tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1);
+  const int wave = tid / WAVE;
+  __shared__ int s_key[NW];
+  __shared__ V s_val[NW][REDN];
+  __shared__ int s_trail_row;
+  __shared__ V s_trail_val[REDN];
   Pack<V, AGG> acc;
   zero(acc);
-  for (int t = first; t < num_tiles; t += stride) {
+  const int first_chunk = SINGLE ? 0 : (int)blockIdx.x * BLOCK;
+  const int chunk_step = SINGLE ? BLOCK : num_tiles;  // not SINGLE: one chunk per block
+  for (int chunk = first_chunk; chunk < num_tiles; chunk += chunk_step) {
+    const int t = chunk + tid;
+    const bool valid = t < num_tiles;
     if constexpr (RED > 0) {
-      const int row = carry_row[t];
-      if (row >= 0 && !(t > 0 && carry_row[t - 1] == row)) {  // first tile of this row's run
-        Pack<V, RED> sum;
+      const int row = valid ? carry_row[t] : -1;
+      const int next_row = (valid && t + 1 < num_tiles) ? carry_row[t + 1] : -2;
+      V run[REDN];
 #pragma unroll
-        for (int c = 0; c < RED; ++c) sum.v[c] = carry_val[(size_t)t * RED + c];
-        for (int u = t + 1; u < num_tiles && carry_row[u] == row; ++u) {
+      for (int c = 0; c < RED; ++c) run[c] = (row >= 0) ? carry_val[(size_t)t * RED + c] : V(0);
+      // does the chunk start inside a run that an earlier chunk owns?
+      const int chunk_first_row = carry_row[chunk];
+      const bool leading_continues = chunk > 0 && chunk_first_row >= 0 && carry_row[chunk - 1] == chunk_first_row;
+      // segmented inclusive sums over the chunk, keyed by row (equal rows are contiguous)
+      wave_segmented_inclusive_sum<V, REDN>(row, run);
+      if (tid == 0) s_trail_row = -1;
+      if (lane == WAVE - 1) {
+        s_key[wave] = row;
 #pragma unroll
-          for (int c = 0; c < RED; ++c) sum.v[c] += carry_val[(size_t)u * RED + c];
-        }
-        G::add_row(p, row, sum);
+        for (int c = 0; c < RED; ++c) s_val[wave][c] = run[c];
       }
+      __syncthreads();
+      {
+        int pk = -3;
+        V pv[REDN];
+#pragma unroll
+        for (int c = 0; c < RED; ++c) pv[c] = V(0);
+        for (int w = 0; w < NW - 1; ++w) {
+          if (w < wave) {
+            const int k = s_key[w];
+#pragma unroll
+            for (int c = 0; c < RED; ++c) pv[c] = (k == pk) ? static_cast<V>(pv[c] + s_val[w][c]) : s_val[w][c];
+            pk = k;
+          }
+        }
+        if (wave > 0 && row >= 0 && row == pk) {  // my run began in an earlier wavefront of this chunk
+#pragma unroll
+          for (int c = 0; c < RED; ++c) run[c] += pv[c];
+        }
+      }
+      const bool mine = row >= 0 && !(leading_continues && row == chunk_first_row);
+      const bool part_end = next_row != row || tid == BLOCK - 1;  // last tile of the run inside this chunk
+      if (mine && part_end) {
+        if (next_row != row) {  // the run ends here
+          Pack<V, RED> sum;
+#pragma unroll
+          for (int c = 0; c < RED; ++c) sum.v[c] = run[c];
+          G::add_row(p, row, sum);
+        } else {  // it goes on in the following chunks: the block finishes it together
+          s_trail_row = row;
+#pragma unroll
+          for (int c = 0; c < RED; ++c) s_trail_val[c] = run[c];
+        }
+      }
+      __syncthreads();
+      const int trail_row = s_trail_row;
+      if (trail_row >= 0) {  // uniform
+        V ext[REDN];
+#pragma unroll
+        for (int c = 0; c < RED; ++c) ext[c] = V(0);
+        for (int base = chunk + BLOCK; base < num_tiles; base += BLOCK) {
+          const int u = base + tid;
+          const bool same = u < num_tiles && carry_row[u] == trail_row;
+          if (same) {
+#pragma unroll
+            for (int c = 0; c < RED; ++c) ext[c] += carry_val[(size_t)u * RED + c];
+          }
+          if (!__syncthreads_and(same ? 1 : 0)) break;  // the run is contiguous: a mismatch ends it
+        }
+        wave_sum_to_last_lane<V, REDN>(ext);
+        __syncthreads();  // s_val is free again
+        if (lane == WAVE - 1) {
+#pragma unroll
+          for (int c = 0; c < RED; ++c) s_val[wave][c] = ext[c];
+        }
+        __syncthreads();
+        if (tid == 0) {
+          Pack<V, RED> sum;
+#pragma unroll
+          for (int c = 0; c < RED; ++c) {
+            V x = s_trail_val[c];
+            for (int w = 0; w < NW; ++w) x += s_val[w][c];
+            sum.v[c] = x;
+          }
+          G::add_row(p, trail_row, sum);
+        }
+      }
+      __syncthreads();  // before the next chunk reuses the shared arrays
     }
     if constexpr (AGG > 0) {
+      if (valid) {
 #pragma unroll
-      for (int w = 0; w < PARTS_PER_TILE; ++w) {
+        for (int w = 0; w < PARTS_PER_TILE; ++w) {
 #pragma unroll
-        for (int c = 0; c < AGG; ++c) acc.v[c] += agg_partials[((size_t)t * PARTS_PER_TILE + w) * AGG + c];
+          for (int c = 0; c < AGG; ++c) acc.v[c] += agg_partials[((size_t)t * PARTS_PER_TILE + w) * AGG + c];
+        }
       }
     }
   }
   if constexpr (AGG > 0) {
     __shared__ V s_wave_agg[NW][AGG];
     wave_sum_to_last_lane<V, AGG>(acc.v);
-    if ((threadIdx.x & (WAVE - 1)) == WAVE - 1) {
+    if (lane == WAVE - 1) {
 #pragma unroll
-      for (int c = 0; c < AGG; ++c) s_wave_agg[threadIdx.x / WAVE][c] = acc.v[c];
+      for (int c = 0; c < AGG; ++c) s_wave_agg[wave][c] = acc.v[c];
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (tid == 0) {
       Pack<V, AGG> total;
 #pragma unroll
       for (int c = 0; c < AGG; ++c) {

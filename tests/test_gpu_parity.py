@@ -533,3 +533,35 @@ def test_launches_on_two_streams_do_not_share_scratch():
     dev = torch.device("cuda", torch.cuda.current_device())
     a, b = (ext.workspace_of(dev, st) for st in streams)
     assert a is not None and b is not None and a.data_ptr() != b.data_ptr()
+
+
+@pytest.mark.parametrize("case", ["one_block_walks_the_chunks", "a_block_per_chunk"])
+def test_rows_that_span_hundreds_of_tiles(case):
+    """A row of millions of non-zeros carries into the same row from hundreds of consecutive tiles.  The fix-up
+    folds such a run with the whole block (in a fixed order), also across the chunks of tiles a block handles:
+    runs longer than a chunk, runs that start in the middle of a chunk, in launches small enough for one fix-up
+    block (chunks of 1024 tiles) and in larger ones (a block per 256 tiles)."""
+    rng = case_rng("hub_rows", case)
+    if case == "one_block_walks_the_chunks":
+        lens = np.concatenate([rng.integers(0, 9, 3000), [2_600_000], rng.integers(0, 9, 500), [700_000],
+                               rng.integers(0, 9, 3000)])
+    else:
+        lens = np.concatenate([rng.integers(0, 9, 400_000), [1_500_000], rng.integers(2, 7, 900_000), [600_000, 0, 5],
+                               rng.integers(0, 9, 400_000)])
+    row_ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    # float64: over a million float32 terms the reference's own sequential sums are off by more than 1e-5
+    for name, dtype in (("csr_spmv", np.float64), ("swe_rusanov", np.float64)):
+        tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get(name), dtype, rng, row_ptr=row_ptr)
+        ext = load_named(name, build_if_missing=False)
+        tiles = ctypes_tiling(ext, np.dtype(dtype).name, nr, ne)
+        print(f"case hub rows {case} {name} {np.dtype(dtype).name} rows={nr} ne={ne} tiles={tiles}", flush=True)
+        assert (tiles <= 4096) == (case == "one_block_walks_the_chunks")
+        check_against_oracle(name, tensors, row_ptr, nr, nc, dtype)
+
+
+def ctypes_tiling(ext, dtype, num_rows, ne):
+    import ctypes
+    from flexspmv_amd.binding import DTYPE_CODES
+    out = (ctypes.c_int32 * 6)()
+    assert ext._lib.flexspmv_tiling(DTYPE_CODES[dtype], num_rows, ne, out) == 0
+    return int(out[0])
