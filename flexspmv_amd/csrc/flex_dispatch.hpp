@@ -8,6 +8,7 @@
 // protocol, and the caller owns the scratch so nothing is allocated per launch.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
 
@@ -34,7 +35,10 @@ inline int fail_hip(hipError_t e, const char* where) {
   return (int)e;
 }
 
-// HIP events that bracket the dominant kernel of a launch made with FLEXSPMV_FLAG_TIME_KERNEL.
+// HIP events of the dominant kernel of a launch made with FLEXSPMV_FLAG_TIME_KERNEL.  They are attached to the
+// kernel's own dispatch (hipExtLaunchKernelGGL), so their difference is the kernel's execution time on
+// the launch stream - events recorded before and after the launch also count the dispatch of the kernel
+// and of the two event markers, 5 - 8 us on a 300 us kernel.
 struct KernelTimer {
   hipEvent_t start = nullptr, stop = nullptr;
   bool armed = false;
@@ -265,7 +269,7 @@ struct Dispatch {
     static thread_local GridCache grid_cache;  // one per kernel instantiation and host thread
     hipStream_t stream = (hipStream_t)a->stream;
     const bool timed = (a->flags & FLEXSPMV_FLAG_TIME_KERNEL) != 0 && g_timer.ready();
-    g_timer.armed = false;
+    if (timed) g_timer.armed = false;  // untimed launches leave the last timed kernel's events readable
     V* partials = (V*)(ws + l.off_partials);
     const int nnz = (int)a->ne;
 
@@ -282,7 +286,6 @@ struct Dispatch {
         hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(SEARCH_BLOCK), 0, stream, l.tiling, row_end,
                            num_rows, nnz, coords);
       }
-      if (timed) (void)hipEventRecord(g_timer.start, stream);
 #ifdef FLEX_TUNE_PERSISTENT
       const int reduce_grid = l.num_tiles < 256 * FLEX_TUNE_PERSISTENT ? l.num_tiles : 256 * FLEX_TUNE_PERSISTENT;
 #else
@@ -290,9 +293,15 @@ struct Dispatch {
 #endif
       const int2* table = l.search_in_blocks ? nullptr : coords;
       int2* table_out = (l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_KEEP_TILES) != 0) ? coords : nullptr;
-      hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(reduce_grid), dim3(BLOCK), 0, stream, table, l.tiling,
-                         num_rows, row_end, nnz, p, carry_row, carry_val, partials, table_out);
-      if (timed) g_timer.armed = (hipEventRecord(g_timer.stop, stream) == hipSuccess);
+      if (timed) {
+        hipExtLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(reduce_grid), dim3(BLOCK), 0, stream, g_timer.start,
+                              g_timer.stop, 0, table, l.tiling, num_rows, row_end, nnz, p, carry_row, carry_val, partials,
+                              table_out);
+        g_timer.armed = true;
+      } else {
+        hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(reduce_grid), dim3(BLOCK), 0, stream, table, l.tiling,
+                           num_rows, row_end, nnz, p, carry_row, carry_val, partials, table_out);
+      }
       V* block_partials = (V*)(ws + l.off_block_partials);
       if (l.single_fixup) {
         hipLaunchKernelGGL((fixup_kernel<G, SINGLE_FIXUP_BLOCK, BLOCK / WAVE, true>), dim3(1), dim3(SINGLE_FIXUP_BLOCK), 0,
@@ -310,10 +319,14 @@ struct Dispatch {
     } else {
       int grid = resident_grid(flat_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
       if (grid > l.num_tiles) grid = l.num_tiles;
-      if (timed) (void)hipEventRecord(g_timer.start, stream);
-      hipLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream, p, nnz,
-                         l.num_tiles, partials);
-      if (timed) g_timer.armed = (hipEventRecord(g_timer.stop, stream) == hipSuccess);
+      if (timed) {
+        hipExtLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream, g_timer.start,
+                              g_timer.stop, 0, p, nnz, l.num_tiles, partials);
+        g_timer.armed = true;
+      } else {
+        hipLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream, p, nnz, l.num_tiles,
+                           partials);
+      }
       if (G::AGG_WIDTH > 0) {
         hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
                            (const V*)partials, grid);

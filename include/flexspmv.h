@@ -40,7 +40,7 @@ extern "C" {
 #define FLEXSPMV_STATIC_SCRATCH_BYTES (4u << 20)
 
 /* flexspmv_launch_args.flags */
-#define FLEXSPMV_FLAG_TIME_KERNEL 1u /* bracket the dominant kernel with HIP events on args->stream */
+#define FLEXSPMV_FLAG_TIME_KERNEL 1u /* attach HIP events to the dominant kernel's dispatch on args->stream */
 /* Skip the tile search: the caller guarantees that the previous launch of this library with this
  * workspace completed, used the same dtype, num_rows, ne and the same, unmodified row_end_offsets, and
  * that nothing else wrote to the workspace since.  The tile table left in the workspace by that launch
@@ -132,7 +132,7 @@ const char* flexspmv_last_error(void);
 
 /* Duration in milliseconds of the dominant kernel (the reducer kernel, or the flat kernel of an
  * aggregator / map-only library) of the calling thread's most recent flexspmv_launch that carried
- * FLEXSPMV_FLAG_TIME_KERNEL.  Blocks until that kernel has finished.  Returns FLEXSPMV_OK, or
+ * FLEXSPMV_FLAG_TIME_KERNEL (launches without the flag made since do not disturb it).  Blocks until that kernel has finished.  Returns FLEXSPMV_OK, or
  * FLEXSPMV_ERR_BAD_ARGUMENT when no such launch was made. */
 int flexspmv_last_kernel_ms(float* ms);
 
