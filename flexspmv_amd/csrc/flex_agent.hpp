@@ -270,6 +270,20 @@ inline int grid_for_tiles(int num_tiles, int xcd_shift) {
   return xcd_shift == 0 ? num_tiles : (num_tiles + window - 1) / window * window;
 }
 
+// Neighbouring edges a thread takes per first-level load on launches with short, regular rows: as many
+// (a power of two, at most 4 and at most IPT) as keep what it fetches for them within 48 bytes.  Plain SpMV
+// in float64 (12 bytes per edge): 4 - its 8- and 4-byte loads become 16-byte loads, 3 % on Poisson 256^3.
+// The shallow-water map (28 bytes per edge, 16 of them one load already) stays at 1: 2 measured 2 % slower.
+// Power-law launches always use 1: their map runs in coalesced edge order, where neighbouring lanes should
+// hold neighbouring edges (R-MAT: 370 us with 2 or 4 against 344).
+template <class G, int IPT>
+constexpr int edges_per_load() {
+  constexpr int bytes = G::FETCH_VALUES * (int)sizeof(typename G::Value) + G::FETCH_INDICES * 4;
+  int epl = 1;
+  while (epl * 2 <= 4 && epl * 2 <= IPT && IPT % (epl * 2) == 0 && epl * 2 * bytes <= 48) epl *= 2;
+  return epl;
+}
+
 // ----------------------------------------------------------------------------------------------
 // Reducer kernel.  One block per merge tile of at most BLOCK*IPT merge items (R row ends + Z non-zeros),
 // found by the tile search.  Blocks are small and independent; overlap of one block's memory waits
@@ -297,7 +311,7 @@ inline int grid_for_tiles(int num_tiles, int xcd_shift) {
 // lanes read a clamped address, and per-item work is predicated.  Every row is written exactly once;
 // the tile's open last row becomes a carry record for fixup_kernel.
 // ----------------------------------------------------------------------------------------------
-template <class G, int BLOCK, int IPT>
+template <class G, int BLOCK, int IPT, int EPL>
 __device__ __forceinline__ void
 reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hint, const int num_rows,
             const int* __restrict__ row_end, const int nnz, const typename G::Params& p, int* __restrict__ carry_row,
@@ -360,12 +374,40 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   const int last_edge = nnz - 1;
   const int last_row = num_rows - 1;
 
+  // Which edge of the tile a thread's k-th first-level load takes: EPL neighbouring edges per thread (its
+  // loads of them merge into wider ones: 16 bytes per lane instead of 4 or 8), threads side by side.
+  static_assert(EPL >= 1 && IPT % EPL == 0, "edges per load must divide the items per thread");
+  auto slot_of = [&](const int k) { return (k / EPL) * (EPL * BLOCK) + tid * EPL + (k % EPL); };
+
   // 1: first-level loads.  A tile holds Z <= TILE non-zeros; lanes past Z re-read the tile's last
   // edge (one cache line, no extra traffic) instead of running into the next tile's edges.
   Fetch f[IPT];
   const int e_last = min(y0 + max(Z - 1, 0), last_edge);
 #pragma unroll
-  for (int k = 0; k < IPT; ++k) G::fetch(p, min(y0 + tid + k * BLOCK, e_last), f[k]);
+  for (int k = 0; k < IPT; k += EPL) {
+    if constexpr (EPL == 1) {
+      G::fetch(p, min(y0 + slot_of(k), e_last), f[k]);
+    } else {
+      // EPL neighbouring edges from one base address, so that the loads merge.  A group that would run past
+      // the end of the edge list (last tile only; the host launches this variant only when there are at
+      // least EPL edges) is read from the last EPL edges instead and shifted into place, so that slot j
+      // still holds edge min(y0 + j, last edge).  A group past the tile's own edges simply reads the next
+      // tile's: those slots are never used.
+      const int want = y0 + slot_of(k);
+      const int e0 = min(want, last_edge - (EPL - 1));
+      const int shift = want - e0;  // 0 except at the very end of the edge list
+      Fetch g[EPL];
+#pragma unroll
+      for (int q = 0; q < EPL; ++q) G::fetch(p, e0 + q, g[q]);
+#pragma unroll
+      for (int q = 0; q < EPL; ++q) {
+        f[k + q] = g[EPL - 1];
+#pragma unroll
+        for (int r = q; r < EPL - 1; ++r)
+          if (q + shift == r) f[k + q] = g[r];
+      }
+    }
+  }
   // ... and of the rows: thread tid holds the end of tile row tid, the first wavefront also the end
   // of row BLOCK + tid; lane 0 of each wavefront fetches the end of the row before its first one,
   // the other lanes get it from their neighbour, so every thread knows where its row starts.
@@ -389,7 +431,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   // 2: hand-over through LDS, in coalesced order.  Every slot of the tile is written (slots past Z hold
   // copies of the tile's last edge), so a clamped read always finds a real edge.
 #pragma unroll
-  for (int k = 0; k < IPT; ++k) G::template put<TILE>(f[k], s_fv, s_fi, k * BLOCK + tid);
+  for (int k = 0; k < IPT; ++k) G::template put<TILE>(f[k], s_fv, s_fi, slot_of(k));
 
   // vote - can every row of this tile be summed by one thread?  Row i of the tile spans the
   // tile-relative non-zeros [end(i-1), end(i)), with end(-1) = 0 and, for the row still open at the
@@ -516,7 +558,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
         for (int k = 0; k < MERGE_CHUNK; ++k) G::gather(p, f[k0 + k], g[k]);
 #pragma unroll
         for (int k = 0; k < MERGE_CHUNK; ++k) {
-          const int j = (k0 + k) * BLOCK + tid;
+          const int j = slot_of(k0 + k);
           if (G::EDGE_PURE || j < Z) {
             Pack<V, RED> dt;
             Pack<V, AGG> da;
@@ -719,7 +761,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
 // With FLEX_TUNE_PERSISTENT (tuning switch) a launch has at most that many blocks per CU; each walks
 // tiles blockIdx.x, blockIdx.x + gridDim.x, ... and reads the coordinates of its next tile while it
 // works on the current one.
-template <class G, int BLOCK, int IPT>
+template <class G, int BLOCK, int IPT, int EPL>
 __global__ void __launch_bounds__(BLOCK)
 reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_rows, const int* __restrict__ row_end,
               const int nnz, const typename G::Params p, int* __restrict__ carry_row,
@@ -738,7 +780,7 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
       n0 = coords[next];
       n1 = coords[next + 1];
     }
-    reduce_tile<G, BLOCK, IPT>(tile, c0, c1, tl.row_group, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
+    reduce_tile<G, BLOCK, IPT, EPL>(tile, c0, c1, tl.row_group, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
     if (!more) break;
     __syncthreads();  // the tile's LDS is free again
     tile = next;
@@ -782,7 +824,7 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
       if (tile == num_tiles - 1) coords_out[num_tiles] = c1;
     }
   }
-  reduce_tile<G, BLOCK, IPT>(tile, c0, c1, tl.row_group, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
+  reduce_tile<G, BLOCK, IPT, EPL>(tile, c0, c1, tl.row_group, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
 #endif
 }
 

@@ -293,15 +293,21 @@ struct Dispatch {
 #endif
       const int2* table = l.search_in_blocks ? nullptr : coords;
       int2* table_out = (l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_KEEP_TILES) != 0) ? coords : nullptr;
-      if (timed) {
-        hipExtLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(reduce_grid), dim3(BLOCK), 0, stream, g_timer.start,
-                              g_timer.stop, 0, table, l.tiling, num_rows, row_end, nnz, p, carry_row, carry_val, partials,
-                              table_out);
-        g_timer.armed = true;
-      } else {
-        hipLaunchKernelGGL((reduce_kernel<G, BLOCK, IPT>), dim3(reduce_grid), dim3(BLOCK), 0, stream, table, l.tiling,
-                           num_rows, row_end, nnz, p, carry_row, carry_val, partials, table_out);
-      }
+      // launches with short regular rows (row-snapped tiles) take several neighbouring edges per load
+      constexpr int EPL = edges_per_load<G, IPT>();
+      const bool wide_loads = EPL > 1 && l.tiling.snap_slack > 0 && nnz >= EPL;
+      auto launch_reducer = [&](auto kernel) {
+        if (timed) {
+          hipExtLaunchKernelGGL(kernel, dim3(reduce_grid), dim3(BLOCK), 0, stream, g_timer.start, g_timer.stop, 0, table,
+                                l.tiling, num_rows, row_end, nnz, p, carry_row, carry_val, partials, table_out);
+          g_timer.armed = true;
+        } else {
+          hipLaunchKernelGGL(kernel, dim3(reduce_grid), dim3(BLOCK), 0, stream, table, l.tiling, num_rows, row_end, nnz, p,
+                             carry_row, carry_val, partials, table_out);
+        }
+      };
+      if (wide_loads) launch_reducer(reduce_kernel<G, BLOCK, IPT, EPL>);
+      else launch_reducer(reduce_kernel<G, BLOCK, IPT, 1>);
       V* block_partials = (V*)(ws + l.off_block_partials);
       if (l.single_fixup) {
         hipLaunchKernelGGL((fixup_kernel<G, SINGLE_FIXUP_BLOCK, BLOCK / WAVE, true>), dim3(1), dim3(SINGLE_FIXUP_BLOCK), 0,
