@@ -418,7 +418,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
     re = row_end[r1];
     if constexpr (ROW > 0) G::load_row(p, r1, rowv);
     if (lane == 0 && tid > 0) prev_lane0 = row_end[min(x0 + tid - 1, last_row)];
-    if (wave == 0) {
+    if (wave == 0 && R + 1 > BLOCK) {  // uniform: only tiles with more rows than threads need a second pass
       const int r2 = min(x0 + BLOCK + tid, min(x0 + R, last_row));
       re2 = row_end[r2];
       if constexpr (ROW > 0) G::load_row(p, r2, rowv2);
