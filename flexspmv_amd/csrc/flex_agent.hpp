@@ -922,7 +922,49 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
   zero(acc);
   const int first_chunk = SINGLE ? 0 : (int)blockIdx.x * BLOCK;
   const int chunk_step = SINGLE ? BLOCK : num_tiles;  // not SINGLE: one chunk per block
-  for (int chunk = first_chunk; chunk < num_tiles; chunk += chunk_step) {
+  // One block for all chunks: one pass with all loads in flight together sums the aggregator partials and
+  // looks whether any run is longer than a tile.  If none is (always on row-snapped launches, where no
+  // tile carries at all), every carry goes to its row as it is and the chunk loop below is skipped.
+  bool may_have_runs = true;
+  bool partials_done = false;
+  if constexpr (SINGLE) {
+    constexpr int KEPT = 4;  // carries a thread keeps in registers between the two phases
+    int kept_row[KEPT];
+    bool multi = false;
+    for (int i = 0, t = tid; t < num_tiles; ++i, t += BLOCK) {
+      if constexpr (RED > 0) {
+        const int row = carry_row[t];
+        const int next_row = (t + 1 < num_tiles) ? carry_row[t + 1] : -2;
+        multi |= (row >= 0 && next_row == row);
+        if (i < KEPT) kept_row[i] = row;
+      }
+      if constexpr (AGG > 0) {
+#pragma unroll
+        for (int w = 0; w < PARTS_PER_TILE; ++w) {
+#pragma unroll
+          for (int c = 0; c < AGG; ++c) acc.v[c] += agg_partials[((size_t)t * PARTS_PER_TILE + w) * AGG + c];
+        }
+      }
+    }
+    partials_done = true;
+    if constexpr (RED > 0) {
+      may_have_runs = __syncthreads_or(multi ? 1 : 0) != 0;
+      if (!may_have_runs) {
+        for (int i = 0, t = tid; t < num_tiles; ++i, t += BLOCK) {
+          const int row = (i < KEPT) ? kept_row[i] : carry_row[t];
+          if (row >= 0 && !(t > 0 && carry_row[t - 1] == row)) {
+            Pack<V, RED> sum;
+#pragma unroll
+            for (int c = 0; c < RED; ++c) sum.v[c] = carry_val[(size_t)t * RED + c];
+            G::add_row(p, row, sum);
+          }
+        }
+      }
+    } else {
+      may_have_runs = false;
+    }
+  }
+  for (int chunk = first_chunk; chunk < num_tiles && (!SINGLE || may_have_runs); chunk += chunk_step) {
     const int t = chunk + tid;
     const bool valid = t < num_tiles;
     if constexpr (RED > 0) {
@@ -931,87 +973,98 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
       V run[REDN];
 #pragma unroll
       for (int c = 0; c < RED; ++c) run[c] = (row >= 0) ? carry_val[(size_t)t * RED + c] : V(0);
-      // does the chunk start inside a run that an earlier chunk owns?
-      const int chunk_first_row = carry_row[chunk];
-      const bool leading_continues = chunk > 0 && chunk_first_row >= 0 && carry_row[chunk - 1] == chunk_first_row;
-      // segmented inclusive sums over the chunk, keyed by row (equal rows are contiguous)
-      wave_segmented_inclusive_sum<V, REDN>(row, run);
-      if (tid == 0) s_trail_row = -1;
-      if (lane == WAVE - 1) {
-        s_key[wave] = row;
-#pragma unroll
-        for (int c = 0; c < RED; ++c) s_val[wave][c] = run[c];
-      }
-      __syncthreads();
-      {
-        int pk = -3;
-        V pv[REDN];
-#pragma unroll
-        for (int c = 0; c < RED; ++c) pv[c] = V(0);
-        for (int w = 0; w < NW - 1; ++w) {
-          if (w < wave) {
-            const int k = s_key[w];
-#pragma unroll
-            for (int c = 0; c < RED; ++c) pv[c] = (k == pk) ? static_cast<V>(pv[c] + s_val[w][c]) : s_val[w][c];
-            pk = k;
-          }
-        }
-        if (wave > 0 && row >= 0 && row == pk) {  // my run began in an earlier wavefront of this chunk
-#pragma unroll
-          for (int c = 0; c < RED; ++c) run[c] += pv[c];
-        }
-      }
-      const bool mine = row >= 0 && !(leading_continues && row == chunk_first_row);
-      const bool part_end = next_row != row || tid == BLOCK - 1;  // last tile of the run inside this chunk
-      if (mine && part_end) {
-        if (next_row != row) {  // the run ends here
+      // Most chunks have no run of more than one tile (none at all on row-snapped launches): then a tile's
+      // carry goes to its row as it is, unless the tile continues a run that an earlier chunk owns.
+      if (!may_have_runs || !__syncthreads_or((row >= 0 && next_row == row) ? 1 : 0)) {
+        if (row >= 0 && !(t > 0 && carry_row[t - 1] == row)) {
           Pack<V, RED> sum;
 #pragma unroll
           for (int c = 0; c < RED; ++c) sum.v[c] = run[c];
           G::add_row(p, row, sum);
-        } else {  // it goes on in the following chunks: the block finishes it together
-          s_trail_row = row;
-#pragma unroll
-          for (int c = 0; c < RED; ++c) s_trail_val[c] = run[c];
         }
-      }
-      __syncthreads();
-      const int trail_row = s_trail_row;
-      if (trail_row >= 0) {  // uniform
-        V ext[REDN];
-#pragma unroll
-        for (int c = 0; c < RED; ++c) ext[c] = V(0);
-        for (int base = chunk + BLOCK; base < num_tiles; base += BLOCK) {
-          const int u = base + tid;
-          const bool same = u < num_tiles && carry_row[u] == trail_row;
-          if (same) {
-#pragma unroll
-            for (int c = 0; c < RED; ++c) ext[c] += carry_val[(size_t)u * RED + c];
-          }
-          if (!__syncthreads_and(same ? 1 : 0)) break;  // the run is contiguous: a mismatch ends it
-        }
-        wave_sum_to_last_lane<V, REDN>(ext);
-        __syncthreads();  // s_val is free again
+      } else {
+        // does the chunk start inside a run that an earlier chunk owns?
+        const int chunk_first_row = carry_row[chunk];
+        const bool leading_continues = chunk > 0 && chunk_first_row >= 0 && carry_row[chunk - 1] == chunk_first_row;
+        // segmented inclusive sums over the chunk, keyed by row (equal rows are contiguous)
+        wave_segmented_inclusive_sum<V, REDN>(row, run);
+        if (tid == 0) s_trail_row = -1;
         if (lane == WAVE - 1) {
+          s_key[wave] = row;
 #pragma unroll
-          for (int c = 0; c < RED; ++c) s_val[wave][c] = ext[c];
+          for (int c = 0; c < RED; ++c) s_val[wave][c] = run[c];
         }
         __syncthreads();
-        if (tid == 0) {
-          Pack<V, RED> sum;
+        {
+          int pk = -3;
+          V pv[REDN];
 #pragma unroll
-          for (int c = 0; c < RED; ++c) {
-            V x = s_trail_val[c];
-            for (int w = 0; w < NW; ++w) x += s_val[w][c];
-            sum.v[c] = x;
+          for (int c = 0; c < RED; ++c) pv[c] = V(0);
+          for (int w = 0; w < NW - 1; ++w) {
+            if (w < wave) {
+              const int k = s_key[w];
+#pragma unroll
+              for (int c = 0; c < RED; ++c) pv[c] = (k == pk) ? static_cast<V>(pv[c] + s_val[w][c]) : s_val[w][c];
+              pk = k;
+            }
           }
-          G::add_row(p, trail_row, sum);
+          if (wave > 0 && row >= 0 && row == pk) {  // my run began in an earlier wavefront of this chunk
+#pragma unroll
+            for (int c = 0; c < RED; ++c) run[c] += pv[c];
+          }
         }
+        const bool mine = row >= 0 && !(leading_continues && row == chunk_first_row);
+        const bool part_end = next_row != row || tid == BLOCK - 1;  // last tile of the run inside this chunk
+        if (mine && part_end) {
+          if (next_row != row) {  // the run ends here
+            Pack<V, RED> sum;
+#pragma unroll
+            for (int c = 0; c < RED; ++c) sum.v[c] = run[c];
+            G::add_row(p, row, sum);
+          } else {  // it goes on in the following chunks: the block finishes it together
+            s_trail_row = row;
+#pragma unroll
+            for (int c = 0; c < RED; ++c) s_trail_val[c] = run[c];
+          }
+        }
+        __syncthreads();
+        const int trail_row = s_trail_row;
+        if (trail_row >= 0) {  // uniform
+          V ext[REDN];
+#pragma unroll
+          for (int c = 0; c < RED; ++c) ext[c] = V(0);
+          for (int base = chunk + BLOCK; base < num_tiles; base += BLOCK) {
+            const int u = base + tid;
+            const bool same = u < num_tiles && carry_row[u] == trail_row;
+            if (same) {
+#pragma unroll
+              for (int c = 0; c < RED; ++c) ext[c] += carry_val[(size_t)u * RED + c];
+            }
+            if (!__syncthreads_and(same ? 1 : 0)) break;  // the run is contiguous: a mismatch ends it
+          }
+          wave_sum_to_last_lane<V, REDN>(ext);
+          __syncthreads();  // s_val is free again
+          if (lane == WAVE - 1) {
+#pragma unroll
+            for (int c = 0; c < RED; ++c) s_val[wave][c] = ext[c];
+          }
+          __syncthreads();
+          if (tid == 0) {
+            Pack<V, RED> sum;
+#pragma unroll
+            for (int c = 0; c < RED; ++c) {
+              V x = s_trail_val[c];
+              for (int w = 0; w < NW; ++w) x += s_val[w][c];
+              sum.v[c] = x;
+            }
+            G::add_row(p, trail_row, sum);
+          }
+        }
+        __syncthreads();  // before the next chunk reuses the shared arrays
       }
-      __syncthreads();  // before the next chunk reuses the shared arrays
     }
     if constexpr (AGG > 0) {
-      if (valid) {
+      if (valid && !partials_done) {
 #pragma unroll
         for (int w = 0; w < PARTS_PER_TILE; ++w) {
 #pragma unroll
