@@ -174,6 +174,9 @@ struct Dispatch {
 #endif
       }
     }
+#ifdef FLEX_TUNE_NOMINAL  // tuning switch: merge items per tile
+    if (FLEX_TUNE_NOMINAL <= TILE - t.snap_slack) t.nominal = FLEX_TUNE_NOMINAL;
+#endif
     const int64_t items = REDUCER ? num_rows + ne : ne;
     t.num_tiles = (int)((items + t.nominal - 1) / t.nominal);
     return t;
