@@ -89,16 +89,20 @@ def time_workload(w, steps, warmup):
     # enough to bring the clocks back up.  The pause before it lets the worker threads of the host-side
     # generators (numpy / torch CPU kernels), which spin for a while after their last parallel region,
     # get out of the launch thread's way.
+    def warm_up():
+        out = None
+        t0 = time.perf_counter()
+        done = 0
+        while done < max(warmup, 1) or time.perf_counter() - t0 < 0.03:
+            out = ext.merged_spmv_launch(*args)
+            done += 1
+            if done % 16 == 0:
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        return out
+
     time.sleep(0.3)
-    outs = None
-    t0 = time.perf_counter()
-    done = 0
-    while done < max(warmup, 1) or time.perf_counter() - t0 < 0.03:
-        outs = ext.merged_spmv_launch(*args)
-        done += 1
-        if done % 16 == 0:
-            torch.cuda.synchronize()
-    torch.cuda.synchronize()
+    outs = warm_up()
 
     # the timed region: exactly K launches between two synchronisations
     t0 = time.perf_counter()
@@ -123,8 +127,7 @@ def time_workload(w, steps, warmup):
     ms_per_step_reuse = None
     if ext.signature["has_reducer"]:
         ext.reuse_tiles = True
-        ext.merged_spmv_launch(*args)
-        torch.cuda.synchronize()
+        warm_up()   # the launches one by one above let the clocks drop again
         t0 = time.perf_counter()
         for _ in range(steps):
             outs_reuse = ext.merged_spmv_launch(*args)

@@ -294,8 +294,11 @@ struct Dispatch {
 #else
       const int reduce_grid = grid_for_tiles(l.num_tiles, l.tiling.xcd_shift);
 #endif
-      const int2* table = l.search_in_blocks ? nullptr : coords;
-      int2* table_out = (l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_KEEP_TILES) != 0) ? coords : nullptr;
+      // Small launches: the reducer blocks search their own boundaries and leave them in the table on the
+      // way (one 8-byte store per block), so that a later launch that may reuse the table skips the search.
+      const bool search_here = l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0;
+      const int2* table = search_here ? nullptr : coords;
+      int2* table_out = search_here ? coords : nullptr;
       // launches with short regular rows (row-snapped tiles) take several neighbouring edges per load
       constexpr int EPL = edges_per_load<G, IPT>();
       const bool wide_loads = EPL > 1 && l.tiling.snap_slack > 0 && nnz >= EPL;

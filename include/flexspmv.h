@@ -47,10 +47,11 @@ extern "C" {
  * is then reused (the reference recomputes it on every call, include/merged_spmv_kernels.cuh:60-99;
  * a solver iterating on a fixed sparsity pattern needs it once). */
 #define FLEXSPMV_FLAG_REUSE_TILES 2u
-/* Leave the tile table (int32 pairs (rows, non-zeros) for tile boundaries 0 .. num_tiles, at the start
- * of the workspace) behind even when the launch is small enough for the reducer blocks to search their
- * own boundaries and would not write it.  A debugging aid: the table of any launch can be read back
- * and compared with a CPU merge-path search (see flexspmv_tiling for the diagonals). */
+/* Every launch of a library with a reducer leaves its tile table (int32 pairs (rows, non-zeros) for tile
+ * boundaries 0 .. num_tiles) at the start of the workspace: large launches from the search kernel, small
+ * ones from the reducer blocks that search their own boundaries.  It can be read back and compared with
+ * a CPU merge-path search (see flexspmv_tiling for the diagonals).  This flag is accepted and changes
+ * nothing (it used to ask small launches for the table). */
 #define FLEXSPMV_FLAG_KEEP_TILES 4u
 
 /* Value types a library may have been generated for (flexspmv_launch_args.dtype). */

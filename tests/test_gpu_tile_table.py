@@ -18,7 +18,7 @@ torch = pytest.importorskip("torch")
 
 from flexspmv_amd import graphs
 from flexspmv_amd import workloads as W
-from flexspmv_amd.binding import DTYPE_CODES, FLAG_KEEP_TILES, load_named
+from flexspmv_amd.binding import DTYPE_CODES, load_named
 from oracle import build_oracle
 from tests.test_gpu_parity import case_rng
 from tests.util_inputs import STRUCTURES, make_inputs, random_row_structure, row_structure
@@ -64,7 +64,8 @@ def expected_table(merge_lib, row_ptr, tl):
 
 
 def device_table(name, dtype, tensors, row_ptr, num_rows, num_cols):
-    """Launch the library with FLEXSPMV_FLAG_KEEP_TILES and read the table back from its workspace."""
+    """Launch the library and read the tile table back from its workspace (every launch leaves it there:
+    large ones from the search kernel, small ones from the reducer blocks)."""
     ext = load_named(name, build_if_missing=False)
     args = []
     for pname in ext.param_names():
@@ -75,11 +76,7 @@ def device_table(name, dtype, tensors, row_ptr, num_rows, num_cols):
         else:
             t = tensors[pname]
             args.append(t if isinstance(t, torch.Tensor) else torch.from_numpy(np.ascontiguousarray(t)).cuda())
-    ext.extra_flags = FLAG_KEEP_TILES
-    try:
-        ext.merged_spmv_launch(*args)
-    finally:
-        ext.extra_flags = 0
+    ext.merged_spmv_launch(*args)
     torch.cuda.synchronize()
     ne = int(row_ptr[-1])
     tl = tiling_of(ext, dtype, num_rows, ne)
