@@ -75,14 +75,14 @@ def measured_traffic(workload_name: str, kernel: str, policy: str):
     return None
 
 
-def time_workload(w, steps, warmup):
+def time_workload(w, steps, warmup, library=None):
     """GPU leg: returns (result dict, outputs of the last launch as numpy arrays)."""
     import torch
 
     from flexspmv_amd import workloads as W
-    from flexspmv_amd.binding import load_named
+    from flexspmv_amd.binding import HipExtension, load_named
 
-    ext = load_named(w.graph, build_if_missing=False)
+    ext = HipExtension(library) if library else load_named(w.graph, build_if_missing=False)
     args = W.launch_arguments(w, ext.param_names(), "cuda:0")
     # Untimed warm-up: W launches, and in any case launches for 30 ms.  Building a workload keeps the host
     # busy for seconds while the GPU idles and clocks down; a handful of sub-millisecond launches is not
@@ -166,6 +166,8 @@ def time_workload(w, steps, warmup):
         "policy": policy, "policy_tag": f"{policy['block']}x{policy['ipt'][dtype]}",
         "seed": int(w.seed),
     }
+    if library:
+        result["library"] = library
     if ms_per_step_reuse is not None:
         result["ms_per_step_tile_reuse"] = ms_per_step_reuse
         result["gbs_tile_reuse"] = w.algorithmic_bytes / ms_per_step_reuse / 1e6
@@ -259,7 +261,8 @@ def cpu_leg(w, result, outs, cpu_runs):
 
 
 def roofline_of(r):
-    traffic = measured_traffic(r["workload"], r["kernel"], r["policy_tag"])
+    # the traffic table holds the shipped libraries' counters; a variant given with --library has its own
+    traffic = None if r.get("library") else measured_traffic(r["workload"], r["kernel"], r["policy_tag"])
     out = {"bound": "hbm", "achieved": r["kernel_gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
            "frac": r["kernel_gbs"] / HBM_PEAK_GBS, "traffic": traffic["bytes"] if traffic else None,
            "kernel": r["kernel"], "kernel_ms": r["kernel_ms"], "kernel_ms_median": r["kernel_ms_median"],
@@ -347,6 +350,9 @@ def main() -> int:
                          "(default: rmat when the headline is the default Poisson run; 'none' for none)")
     ap.add_argument("--all", action="store_true", help="time all the other four workloads (extra JSON key)")
     ap.add_argument("--cpu-runs", type=int, default=5, help="timed runs of the CPU baseline (0 = skip)")
+    ap.add_argument("--library", default=None,
+                    help="time this library file on the workload instead of the shipped one: a variant of the same "
+                         "sub-graph with another tile shape or tuning switches, from python -m flexspmv_amd.build")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain elementwise copies (dst = src + 1) of 1 GiB, a kernel of known "
                          "traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -369,7 +375,7 @@ def main() -> int:
         w = W.matrix_market_spmv(a.mtx, fused_dot=a.mtx_dot)
     else:
         w = W.WORKLOADS[a.workload](size)
-    head, head_outs = time_workload(w, a.steps, a.warmup)
+    head, head_outs = time_workload(w, a.steps, a.warmup, library=a.library)
     torch.cuda.empty_cache()
     if a.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").fill_(1.0)
@@ -436,6 +442,8 @@ def main() -> int:
     line["roofline"]["launches"] = a.steps
     if a.workload in WORKLOAD_NOTES and a.mtx is None:
         line["config"]["note"] = WORKLOAD_NOTES[a.workload]
+    if a.library:
+        line["config"]["library"] = a.library   # not the shipped library: a variant built for a measurement
     if "ms_per_step_tile_reuse" in head:
         line["with_tile_reuse"] = {"ms_per_step": head["ms_per_step_tile_reuse"], "value": head["gbs_tile_reuse"],
                                    "unit": "GB/s", "note": "tile table of the previous launch reused "

@@ -163,3 +163,35 @@ def compile_formats(force: bool = False) -> str:
     with open(_stamp_path(FORMATS_LIBRARY), "w") as f:
         f.write(_formats_stamp())
     return FORMATS_LIBRARY
+
+
+# ---------------------------------------------------------------------------------------------
+# python -m flexspmv_amd.build --graph NAME [--policy BLOCKxIPT] [-D SWITCH[=VALUE]]... [--out DIR]
+# ---------------------------------------------------------------------------------------------
+VARIANTS_DIR = os.path.join(GENERATED_DIR, "variants")
+
+
+def compile_variant(name: str, policy: Optional[str] = None, defines: Sequence[str] = (),
+                    out_dir: Optional[str] = None) -> str:
+    """Compile a sub-graph of flexspmv_amd.graphs with another tile shape (``"128x4"``: threads per block x
+    merge items per thread) and / or tuning switches (the ``FLEX_TUNE_*`` macros of csrc/), into a
+    directory of its own, for measurements next to the shipped library (``bench.py --library``)."""
+    from . import graphs
+    tag = "-".join([policy or "shipped", *[d.replace("=", "_") for d in defines]])
+    pol = None
+    if policy:
+        block, ipt = (int(v) for v in policy.lower().split("x"))
+        pol = {"block": block, "ipt_f32": ipt, "ipt_f64": ipt}
+    return compile_graph(graphs.get(name), out_dir=os.path.join(out_dir or VARIANTS_DIR, tag), force=True, policy=pol,
+                         extra_flags=[f"-D{d}" for d in defines])
+
+
+if __name__ == "__main__":
+    import argparse
+    ap = argparse.ArgumentParser(description="build a variant of a sub-graph library (tile shape, tuning switches)")
+    ap.add_argument("--graph", required=True)
+    ap.add_argument("--policy", default=None, help="BLOCKxIPT, e.g. 128x4 (default: the generator's choice)")
+    ap.add_argument("-D", dest="defines", action="append", default=[], help="FLEX_TUNE_* switch, e.g. FLEX_TUNE_NT_LOADS")
+    ap.add_argument("--out", default=None, help=f"directory (default {VARIANTS_DIR})")
+    a = ap.parse_args()
+    print(compile_variant(a.graph, a.policy, a.defines, a.out))
