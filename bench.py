@@ -84,16 +84,19 @@ def time_workload(w, steps, warmup, library=None):
 
     ext = HipExtension(library) if library else load_named(w.graph, build_if_missing=False)
     args = W.launch_arguments(w, ext.param_names(), "cuda:0")
-    # Untimed warm-up: W launches, and in any case launches for 30 ms.  Building a workload keeps the host
+    # Untimed warm-up: W launches, and in any case launches for 60 ms.  Building a workload keeps the host
     # busy for seconds while the GPU idles and clocks down; a handful of sub-millisecond launches is not
-    # enough to bring the clocks back up.  The pause before it lets the worker threads of the host-side
+    # enough to bring the clocks back up, and a burst of work that follows an idle stretch - a few
+    # milliseconds are enough - goes through a transient first (rocprofv3's per-dispatch durations of the
+    # Poisson kernel: 307 us for the first 6 launches, 315 - 328 for the next 30, back to 303 - 307 after 17 ms).
+    # Every timed series below therefore starts with the same warm-up.  The pause before it lets the worker threads of the host-side
     # generators (numpy / torch CPU kernels), which spin for a while after their last parallel region,
     # get out of the launch thread's way.
     def warm_up():
         out = None
         t0 = time.perf_counter()
         done = 0
-        while done < max(warmup, 1) or time.perf_counter() - t0 < 0.03:
+        while done < max(warmup, 1) or time.perf_counter() - t0 < 0.06:
             out = ext.merged_spmv_launch(*args)
             done += 1
             if done % 16 == 0:
@@ -140,6 +143,7 @@ def time_workload(w, steps, warmup, library=None):
     # the dominant kernel alone: HIP events attached to its dispatch inside the library, on the launch stream.
     # Every timed launch is issued between two untimed ones, so that the kernel runs in a busy stream as it
     # does in the K-step region (reading its events back idles the GPU for a moment).
+    warm_up()
     kernel_ms = []
     for _ in range(steps):
         ext.merged_spmv_launch(*args)

@@ -137,12 +137,14 @@ __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int
 
 // The same boundary found by a group of W consecutive lanes (W = 8, 16, 32 or 64; all lanes of the group
 // must call it; the result is the same in every lane of the group).  A search by one lane is a chain of
-// dependent loads; here a link of the chain is one load per lane.  Up to three rounds probe W consecutive
-// rows around a guess: first the interpolated position, then that position corrected by the residual at
-// the edge of the window just probed (a Newton step with a W-row window).  Regular matrices end after
-// one or two rounds.  If that fails the bracket shrinks W-fold per round.  The row-start load of a
-// snapped boundary is served from the probes of the round that found the answer when that row is among
-// them.  Result: identical to tile_boundary (same monotone predicate, same rule).
+// dependent loads; here a link of the chain is one load per lane.  Dense rounds probe W consecutive rows
+// around a guess: first the interpolated position, then that position corrected by the residual at the
+// edge of the window just probed (a Newton step with a W-row window and the window's own slope).  Regular
+// matrices end after two or three rounds (the 3-D stencil after four at most; with the global slope and three
+// dense rounds one boundary in seventy needed seven to eleven, and the slowest group is the kernel's time).
+// Where the corrections stop shrinking the bracket is cut W-fold per round instead.  The row-start load
+// of a snapped boundary is served from loads of the round that found the answer.  Result: identical to
+// tile_boundary (same monotone predicate, same rule).
 template <int W>
 __device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end,
                                                     int num_rows, int nnz) {
@@ -162,9 +164,20 @@ __device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, con
   const float inv_slope = (float)num_rows / ((float)num_rows + (float)nnz);
   int guess = (int)((float)diag * inv_slope);
   int win_start = 0, win_end_value = 0;  // window of the round that found the answer, and this lane's probe
+  int win_snap_value = 0;                // ... and what lanes 0 and 1 fetched for the snapping rule in that round
   bool win_valid = false;
+  const bool snapping = tl.snap_slack > 0 && t > 0 && t < tl.num_tiles;
+  // Dense rounds go on for as long as they converge: a round whose correction is not at least four times
+  // smaller than the one before it (rows of very different lengths: no slope predicts them) ends them.
+  // A whole wavefront per boundary (the search inside a reducer block, where every instruction is on the
+  // block's critical path) keeps the plain form: its window is wide enough to hold the row the snapping
+  // rule needs, and the refinements below bought it nothing (spring-mass 100^3: 33.5 us against 31.9).
+  constexpr bool REFINED = W < 64;
+  constexpr int MAX_DENSE_ROUNDS = REFINED ? 6 : 3;
+  long long last_jump = 0;
 #pragma unroll 1
-  for (int round = 0; round < 3 && lo < hi; ++round) {
+  for (int round = 0; round < MAX_DENSE_ROUNDS && lo < hi; ++round) {
+    const int guess_before = guess;
     const int w0 = min(max(guess - LEAD, lo), max(hi - W, lo));  // window [w0, w0 + W) inside [lo, hi)
     const int pos = w0 + glane;
     int end = 0;
@@ -173,24 +186,46 @@ __device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, con
       end = row_end[pos];
       past = end + pos + 1 > diag;
     }
+    // A snapped boundary needs the end of the row before its snap row, which a narrow window rarely holds:
+    // if the answer is in this window, the snap row is one of the first two multiples of the snap width at
+    // or above (w0 rounded down), so lanes 0 and 1 fetch those two values in the same round instead of one
+    // more dependent load afterwards.
+    int snap_value = 0;
+    if (REFINED && snapping && glane < 2) {
+      const int row = (w0 & ~tl.snap_mask) + glane * (tl.snap_mask + 1) - 1;
+      if (row >= 0 && row < num_rows) snap_value = row_end[row];
+    }
     const unsigned long long m = group_ballot(past);
+    // Rows per merge item around here, from the window's own ends, where all of it was probed and its rows
+    // are about as long as the matrix's average: on a regular matrix the next guess then lands on the row
+    // (the global ratio is off by the share of short boundary rows - thousands of rows on a 3-D stencil).
+    float step_slope = inv_slope;
+    if (REFINED && w0 + W <= hi) {
+      const float local = (float)(W - 1) / (float)(from_lane(end, W - 1) - from_lane(end, 0) + (W - 1));
+      if (local > 0.75f * inv_slope && local < 1.33f * inv_slope) step_slope = local;
+    }
     if (m == 0ull) {  // every probed row ends before the diagonal: the answer lies beyond the window
       const int g_last = from_lane(end, W - 1) + (w0 + W - 1) + 1;
       lo = w0 + W;
-      guess = (int)min((long long)lo + (long long)((float)(diag - g_last) * inv_slope), (long long)hi);
+      guess = (int)min((long long)lo + (long long)((float)(diag - g_last) * step_slope), (long long)hi);
     } else {
       const int j = __builtin_ctzll(m);
       if (j > 0 || w0 == lo) {  // rows before w0 + j end before the diagonal, row w0 + j (or hi) does not
         lo = hi = w0 + j;
         win_start = w0;
         win_end_value = end;
+        win_snap_value = snap_value;
         win_valid = true;
       } else {  // the answer is at or before the window's first row
         const int g_first = from_lane(end, 0) + w0 + 1;
         hi = w0;
-        guess = w0 - 1 - (int)((float)(g_first - diag) * inv_slope);
+        guess = w0 - 1 - (int)((float)(g_first - diag) * step_slope);
       }
     }
+    const long long jump = (long long)guess - guess_before;
+    const long long jump_size = jump < 0 ? -jump : jump;
+    if (REFINED && round > 0 && jump_size * 4 > last_jump) break;
+    last_jump = jump_size;
   }
   const int probed_below = min(diag, num_rows);  // window lanes at or beyond this row hold no probe
 #pragma unroll 1
@@ -209,13 +244,16 @@ __device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, con
     hi = new_hi;
   }
   int2 c = make_int2(min(lo, num_rows), diag - lo);
-  if (tl.snap_slack > 0 && t > 0 && t < tl.num_tiles) {
+  if (snapping) {
     const int xs = c.x & ~tl.snap_mask;
     int ys = 0;
     if (xs > 0) {
-      const int src = xs - 1 - win_start;  // lane of the group that probed row xs - 1
+      const int src = xs - 1 - win_start;                                       // lane that probed row xs - 1
+      const int which = (xs - (win_start & ~tl.snap_mask)) / (tl.snap_mask + 1);  // lane that fetched it for the rule
       if (win_valid && src >= 0 && src < W && xs - 1 < probed_below) {
         ys = from_lane(win_end_value, src);
+      } else if (REFINED && win_valid && xs >= (win_start & ~tl.snap_mask) && which < 2) {
+        ys = from_lane(win_snap_value, which);
       } else {
         ys = row_end[xs - 1];
       }
