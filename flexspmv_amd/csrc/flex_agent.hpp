@@ -1071,14 +1071,31 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
           V ext[REDN];
 #pragma unroll
           for (int c = 0; c < RED; ++c) ext[c] = V(0);
-          for (int base = chunk + BLOCK; base < num_tiles; base += BLOCK) {
-            const int u = base + tid;
-            const bool same = u < num_tiles && carry_row[u] == trail_row;
-            if (same) {
+          // EXT_STEP chunks per vote, all their loads in flight together (the values are fetched whether or
+          // not the tile belongs to the run: a load under the test would wait for the row first)
+          constexpr int EXT_STEP = 4;
+          const int last_tile = num_tiles - 1;
+          for (int base = chunk + BLOCK; base < num_tiles; base += EXT_STEP * BLOCK) {
+            int urow[EXT_STEP];
+            V uval[EXT_STEP][REDN];
 #pragma unroll
-              for (int c = 0; c < RED; ++c) ext[c] += carry_val[(size_t)u * RED + c];
+            for (int k = 0; k < EXT_STEP; ++k) {
+              const int u = min(base + k * BLOCK + tid, last_tile);
+              urow[k] = carry_row[u];
+#pragma unroll
+              for (int c = 0; c < RED; ++c) uval[k][c] = carry_val[(size_t)u * RED + c];
             }
-            if (!__syncthreads_and(same ? 1 : 0)) break;  // the run is contiguous: a mismatch ends it
+            bool all_same = true;
+#pragma unroll
+            for (int k = 0; k < EXT_STEP; ++k) {
+              const bool same = base + k * BLOCK + tid < num_tiles && urow[k] == trail_row;
+              all_same &= same;
+              if (same) {
+#pragma unroll
+                for (int c = 0; c < RED; ++c) ext[c] += uval[k][c];
+              }
+            }
+            if (!__syncthreads_and(all_same ? 1 : 0)) break;  // the run is contiguous: a mismatch ends it
           }
           wave_sum_to_last_lane<V, REDN>(ext);
           __syncthreads();  // s_val is free again
