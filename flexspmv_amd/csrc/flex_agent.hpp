@@ -148,7 +148,7 @@ __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int
 template <int W>
 __device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end,
                                                     int num_rows, int nnz) {
-  static_assert(W == 8 || W == 16 || W == 32 || W == 64, "group width");
+  static_assert(W == 2 || W == 4 || W == 8 || W == 16 || W == 32 || W == 64, "group width");
   constexpr int LEAD = (W * 5) / 8;  // rows of the window below the guess (towards the row a snap moves back to)
   const int lane = lane_id();
   const int gbase = lane & ~(W - 1);  // first lane of my group
@@ -273,11 +273,17 @@ __device__ __forceinline__ int2 wave_tile_boundary(int t, const Tiling& tl, cons
 }
 
 // One search per tile boundary: coords[t] is where tile t starts, coords[num_tiles] where the path ends.
-// SEARCH_GROUP lanes per boundary: enough to cut the chain of dependent loads to two or three links, few
-// enough for all boundaries of a large launch to be searched at once.
-constexpr int SEARCH_BLOCK = 256;
+// SEARCH_GROUP lanes per boundary: enough to cut the chain of dependent loads to a few links, few enough
+// for all boundaries of a large launch to be searched at once.  The kernel's time follows the number of
+// threads more than the number of rounds (Poisson 256^3 / R-MAT scale 22, us: 2 lanes 16.9 / 13.8, 4 lanes
+// 9.2 / 11.9, 8 lanes 10.2 / 14.0, 16 lanes 12.1 / 17.5, 32 lanes 17.7 / 22.8; blocks of 64 threads, of 256
+// within 1 us of that).
+#ifndef FLEX_TUNE_SEARCH_BLOCK
+#define FLEX_TUNE_SEARCH_BLOCK 64
+#endif
+constexpr int SEARCH_BLOCK = FLEX_TUNE_SEARCH_BLOCK;
 #ifndef FLEX_TUNE_SEARCH_GROUP
-#define FLEX_TUNE_SEARCH_GROUP 8
+#define FLEX_TUNE_SEARCH_GROUP 4
 #endif
 constexpr int SEARCH_GROUP = FLEX_TUNE_SEARCH_GROUP;
 __global__ void __launch_bounds__(SEARCH_BLOCK)
