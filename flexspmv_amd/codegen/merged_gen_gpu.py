@@ -284,6 +284,12 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         gather_members.append(f"{T} {var};")
         gather_body.append(f"q_g.{var} = {T}(q_p.{target}_ptr + (size_t)q_f.index_{module} * {dim});")
         body.append(f"{T} {var} = q_g.{var};")
+    # every streamed word an array of its own (edge tensors of width 1, index arrays): a tile's slice of it
+    # can then be copied as it lies in memory
+    fetch_contiguous = all(dim == 1 for _, _, dim, _ in kp.fetch_values)
+    value_streams = [f"if (q_w == {first}) return q_p.{target}_ptr;" for _, target, dim, first in kp.fetch_values
+                     if fetch_contiguous]
+    index_streams = [f"if (q_w == {slot}) return q_p.{module}_idx_ptr;" for module, slot in kp.fetch_indices]
     load_row = []
     for var, target, dim, first in kp.row_sources:
         load_row += [f"q_rv.v[{first + i}] = q_p.{target}_ptr[(size_t)q_row * {dim} + {i}];" for i in range(dim)]
@@ -393,6 +399,14 @@ struct Graph {{
 {_indent(fetch_body)}  }}
   static FLEX_DEV void gather(const Params& q_p, const Fetch& q_f, Gather& q_g) {{
 {_indent(gather_body)}  }}
+  // the array behind streamed word q_w, where every streamed word is an array of its own
+  static constexpr bool FETCH_CONTIGUOUS = {'true' if fetch_contiguous else 'false'};
+  static FLEX_DEV const ValueT* value_stream(const Params& q_p, const int q_w) {{
+{_indent(value_streams)}    return nullptr;
+  }}
+  static FLEX_DEV const OffsetT* index_stream(const Params& q_p, const int q_w) {{
+{_indent(index_streams)}    return nullptr;
+  }}
   // hand-over of a tile's fetched data through LDS: word w of tile edge j sits at [w * TILE + j]
   template <int TILE>
   static FLEX_DEV void put(const Fetch& q_f, ValueT* q_sv, OffsetT* q_si, const int q_j) {{

@@ -400,8 +400,8 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   constexpr bool SEPARATE_OUT =
       (size_t)(FV_ELEMS + OUT_ELEMS) * sizeof(V) + (size_t)FIN * TILE * 4 <= (size_t)FLEX_TUNE_SEPARATE_OUT_BYTES;
   constexpr int LDS_ELEMS = SEPARATE_OUT ? FV_ELEMS + OUT_ELEMS : (FV_ELEMS > OUT_ELEMS ? FV_ELEMS : OUT_ELEMS);
-  __shared__ V s_fv[LDS_ELEMS];
-  __shared__ int s_fi[FIN * TILE];
+  __shared__ __attribute__((aligned(16))) V s_fv[LDS_ELEMS];
+  __shared__ __attribute__((aligned(16))) int s_fi[FIN * TILE];
   V* const s_out = SEPARATE_OUT ? s_fv + FV_ELEMS : s_fv;
   __shared__ unsigned s_bits[NWORDS];
   __shared__ int s_vote[NW];
@@ -427,6 +427,44 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   // edge (one cache line, no extra traffic) instead of running into the next tile's edges.
   Fetch f[IPT];
   const int e_last = min(y0 + max(Z - 1, 0), last_edge);
+  // Where every streamed word is an array of its own (edge tensors of width 1, index arrays), the LDS image of
+  // a tile is its slice of those arrays as they lie in memory, and the launches with short regular rows
+  // (EPL > 1) let the loads write it themselves (global_load_lds_dwordx4: 16 bytes per lane, a wavefront's
+  // 1 KB lands contiguously): no landing registers, no LDS stores.  Poisson 256^3: 305.5 us against 307.7.
+  // A tile that reaches past the end of the edge list takes the loads below instead.
+#ifndef FLEX_TUNE_NO_LDS_DIRECT
+  constexpr bool CAN_DIRECT = EPL > 1 && G::FETCH_CONTIGUOUS && TILE % (NW * WAVE * 4) == 0;
+#else
+  constexpr bool CAN_DIRECT = false;
+#endif
+  const bool direct = CAN_DIRECT && (long long)y0 + TILE <= (long long)nnz;  // uniform: every slot is an edge of the list
+  if constexpr (CAN_DIRECT) {
+   if (direct) {
+    constexpr int VPL = 16 / (int)sizeof(V), VPIECE = WAVE * VPL;
+#pragma unroll
+    for (int w = 0; w < FV; ++w) {
+      const V* src = G::value_stream(p, w) + y0;
+#pragma unroll
+      for (int i = 0; i < TILE / VPIECE / NW; ++i) {
+        const int piece = i * NW + wave;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + piece * VPIECE + lane * VPL),
+                                         (__attribute__((address_space(3))) void*)(s_fv + w * TILE + piece * VPIECE), 16, 0, 0);
+      }
+    }
+    constexpr int IPIECE = WAVE * 4;
+#pragma unroll
+    for (int w = 0; w < FI; ++w) {
+      const int* src = G::index_stream(p, w) + y0;
+#pragma unroll
+      for (int i = 0; i < TILE / IPIECE / NW; ++i) {
+        const int piece = i * NW + wave;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + piece * IPIECE + lane * 4),
+                                         (__attribute__((address_space(3))) void*)(s_fi + w * TILE + piece * IPIECE), 16, 0, 0);
+      }
+    }
+   }
+  }
+  if (!direct) {
 #pragma unroll
   for (int k = 0; k < IPT; k += EPL) {
     if constexpr (EPL == 1) {
@@ -452,6 +490,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
       }
     }
   }
+  }
   // ... and of the rows: thread tid holds the end of tile row tid, the first wavefront also the end
   // of row BLOCK + tid; lane 0 of each wavefront fetches the end of the row before its first one,
   // the other lanes get it from their neighbour, so every thread knows where its row starts.
@@ -474,8 +513,12 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
 
   // 2: hand-over through LDS, in coalesced order.  Every slot of the tile is written (slots past Z hold
   // copies of the tile's last edge), so a clamped read always finds a real edge.
+  if (!direct) {
 #pragma unroll
-  for (int k = 0; k < IPT; ++k) G::template put<TILE>(f[k], s_fv, s_fi, slot_of(k));
+    for (int k = 0; k < IPT; ++k) G::template put<TILE>(f[k], s_fv, s_fi, slot_of(k));
+  } else {
+    __builtin_amdgcn_s_waitcnt(0);  // this wavefront's pieces have landed in LDS (the barrier below publishes them)
+  }
 
   // vote - can every row of this tile be summed by one thread?  Row i of the tile spans the
   // tile-relative non-zeros [end(i-1), end(i)), with end(-1) = 0 and, for the row still open at the
@@ -595,6 +638,12 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
     V* const s_x = s_fv;  // MAP_FIRST: contributions [c * TILE + j]; nobody reads s_fv after the vote
     if constexpr (MAP_FIRST) {
       const Pack<V, ROW> no_row{};
+      if constexpr (CAN_DIRECT) {
+        if (direct) {  // the edges went to LDS without passing through registers: take them from there
+#pragma unroll       // (a thread reads its own slots only, and s_x below overwrites just those)
+          for (int k = 0; k < IPT; ++k) G::template get<TILE>(s_fv, s_fi, slot_of(k), f[k]);
+        }
+      }
 #pragma unroll
       for (int k0 = 0; k0 < IPT; k0 += MERGE_CHUNK) {
         Gather g[MERGE_CHUNK];
