@@ -432,7 +432,9 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   // (EPL > 1) let the loads write it themselves (global_load_lds_dwordx4: 16 bytes per lane, a wavefront's
   // 1 KB lands contiguously): no landing registers, no LDS stores.  Poisson 256^3: 305.5 us against 307.7.
   // A tile that reaches past the end of the edge list takes the loads below instead.
-#ifndef FLEX_TUNE_NO_LDS_DIRECT
+#if defined(FLEX_TUNE_LDS_DIRECT_ALL)  // tuning switch: also on launches with long or irregular rows
+  constexpr bool CAN_DIRECT = G::FETCH_CONTIGUOUS && TILE % (NW * WAVE * 4) == 0;
+#elif !defined(FLEX_TUNE_NO_LDS_DIRECT)
   constexpr bool CAN_DIRECT = EPL > 1 && G::FETCH_CONTIGUOUS && TILE % (NW * WAVE * 4) == 0;
 #else
   constexpr bool CAN_DIRECT = false;
