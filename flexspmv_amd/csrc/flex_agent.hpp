@@ -55,7 +55,11 @@ template <typename T> __device__ __forceinline__ T stream_load(const T* p) { ret
 #else
 template <typename T> __device__ __forceinline__ T stream_load(const T* p) { return *p; }
 #endif
-#ifdef FLEX_TUNE_NT_STORES
+#if defined(FLEX_TUNE_ABLATE_STORES)  // ablation (wrong results): what the row outputs cost
+template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) {
+  if (v == T(123456789)) *p = v;
+}
+#elif defined(FLEX_TUNE_NT_STORES)
 template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) { __builtin_nontemporal_store(v, p); }
 #else
 template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) { *p = v; }
