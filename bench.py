@@ -75,7 +75,60 @@ def measured_traffic(workload_name: str, kernel: str, policy: str):
     return None
 
 
-def time_workload(w, steps, warmup, library=None):
+def machine_mix_rate(ext, w, dtype_name, write_bytes, launches=30):
+    """What the memory system delivers for this workload's mix of reads and writes without any arithmetic:
+    the calibration kernel (flexspmv_amd/csrc/flex_calibrate.hip) with one block per tile of the launch, each
+    reading and writing its share of the algorithmic bytes (reads rounded up to 4 KB per tile, writes to 8
+    bytes), tiles dealt to the XCDs as the launch deals them.  Returns a dict for the bench line, or None
+    for sub-graphs without tiles of this kind or when the calibration library is not built."""
+    import ctypes
+
+    import torch
+
+    from flexspmv_amd import build as fbuild
+    from flexspmv_amd.binding import DTYPE_CODES
+    if not ext.signature["has_reducer"] or not os.path.exists(fbuild.CALIBRATE_LIBRARY):
+        return None
+    lib = ctypes.CDLL(fbuild.CALIBRATE_LIBRARY)
+    fn = lib.flexspmv_calibrate_stream_mix
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32,
+                   ctypes.c_int32, ctypes.c_void_p]
+    fn.restype = ctypes.c_int
+    tl = (ctypes.c_int32 * 6)()
+    if ext._lib.flexspmv_tiling(DTYPE_CODES[dtype_name], w.num_rows, w.ne, tl) != 0:
+        return None
+    tiles, snapped = int(tl[0]), int(tl[2]) > 0
+    read_per_tile = -(-(w.algorithmic_bytes - write_bytes) // tiles // 4096) * 4096
+    write_per_tile = min(2048, -(-write_bytes // tiles // 8) * 8)
+    src = torch.ones(tiles * read_per_tile, dtype=torch.uint8, device="cuda:0")
+    dst = torch.empty(tiles * max(write_per_tile, 8), dtype=torch.uint8, device="cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(write, count):
+        """Mean time of `count` launches issued back to back, after 10 untimed ones."""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for i in range(10 + count):
+            if i == 10:
+                e0.record()
+            rc = fn(src.data_ptr(), dst.data_ptr(), tiles, read_per_tile, write, 4 if snapped else 0, 0, stream)
+            if rc != 0:
+                raise RuntimeError(f"calibration kernel failed ({rc})")
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) / count
+
+    for _ in range(2):       # the first series also serves as warm-up of the second
+        ms_mix = run(write_per_tile, launches)
+        ms_read = run(0, launches)
+    moved = tiles * (read_per_tile + write_per_tile)
+    return {"kernel": "one block per tile: 16-byte loads of the tile's share of the reads, 8-byte stores of its "
+                      "share of the writes, no arithmetic (flexspmv_amd/csrc/flex_calibrate.hip)",
+            "tiles": tiles, "read_bytes": tiles * read_per_tile, "write_bytes": tiles * write_per_tile,
+            "ms": ms_mix, "gbs": moved / ms_mix / 1e6,
+            "reads_only_ms": ms_read, "reads_only_gbs": tiles * read_per_tile / ms_read / 1e6}
+
+
+def time_workload(w, steps, warmup, library=None, calibrate=False):
     """GPU leg: returns (result dict, outputs of the last launch as numpy arrays)."""
     import torch
 
@@ -156,6 +209,10 @@ def time_workload(w, steps, warmup, library=None):
     kernel_ms.sort()
 
     dtype = str(next(iter(w.tensors.values())).dtype)
+    machine = None
+    if calibrate:
+        write_bytes = sum(o.numel() * o.element_size() for o in (outs or ()))
+        machine = machine_mix_rate(ext, w, dtype, write_bytes)
     policy = ext.signature["policy"]
     flat = not ext.signature["has_reducer"]
     result = {
@@ -172,6 +229,8 @@ def time_workload(w, steps, warmup, library=None):
     }
     if library:
         result["library"] = library
+    if machine:
+        result["machine"] = machine
     if ms_per_step_reuse is not None:
         result["ms_per_step_tile_reuse"] = ms_per_step_reuse
         result["gbs_tile_reuse"] = w.algorithmic_bytes / ms_per_step_reuse / 1e6
@@ -273,6 +332,11 @@ def roofline_of(r):
            "kernel_ms_min": r["kernel_ms_min"], "launches": None}
     if traffic:
         out["traffic_source"] = traffic["source"]
+    if r.get("machine"):
+        # the same bytes in the same tiles without the arithmetic: how much of the distance to the peak is the machine's
+        out["same_mix_without_arithmetic"] = r["machine"]
+        out["frac_of_same_mix"] = r["machine"]["ms"] * r["algorithmic_bytes"] / (
+            r["machine"]["read_bytes"] + r["machine"]["write_bytes"]) / r["kernel_ms"]
     return out
 
 
@@ -354,6 +418,8 @@ def main() -> int:
                          "(default: rmat when the headline is the default Poisson run; 'none' for none)")
     ap.add_argument("--all", action="store_true", help="time all the other four workloads (extra JSON key)")
     ap.add_argument("--cpu-runs", type=int, default=5, help="timed runs of the CPU baseline (0 = skip)")
+    ap.add_argument("--no-calibration", action="store_true",
+                    help="skip the calibration kernel (the workload's reads and writes without arithmetic)")
     ap.add_argument("--library", default=None,
                     help="time this library file on the workload instead of the shipped one: a variant of the same "
                          "sub-graph with another tile shape or tuning switches, from python -m flexspmv_amd.build")
@@ -379,7 +445,7 @@ def main() -> int:
         w = W.matrix_market_spmv(a.mtx, fused_dot=a.mtx_dot)
     else:
         w = W.WORKLOADS[a.workload](size)
-    head, head_outs = time_workload(w, a.steps, a.warmup, library=a.library)
+    head, head_outs = time_workload(w, a.steps, a.warmup, library=a.library, calibrate=not a.no_calibration)
     torch.cuda.empty_cache()
     if a.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").fill_(1.0)
@@ -398,7 +464,7 @@ def main() -> int:
     pending = []
     for name in other_names:
         wo = W.WORKLOADS[name](DEFAULT_SIZE[name])
-        r, o = time_workload(wo, a.steps, a.warmup)
+        r, o = time_workload(wo, a.steps, a.warmup, calibrate=not a.no_calibration)
         torch.cuda.empty_cache()
         pending.append((name, wo, r, o))
     head = cpu_leg(w, head, head_outs, a.cpu_runs)

@@ -166,6 +166,26 @@ def compile_formats(force: bool = False) -> str:
 
 
 # ---------------------------------------------------------------------------------------------
+# the calibration kernel of bench.py (reads and writes without arithmetic)
+# ---------------------------------------------------------------------------------------------
+CALIBRATE_SOURCE = os.path.join(CSRC_DIR, "flex_calibrate.hip")
+CALIBRATE_LIBRARY = os.path.join(GENERATED_DIR, "libflexspmv_calibrate.so")
+
+
+def compile_calibrate(force: bool = False) -> str:
+    """Compile csrc/flex_calibrate.hip into _generated/libflexspmv_calibrate.so; returns its path."""
+    if (not force and os.path.exists(CALIBRATE_LIBRARY)
+            and os.path.getmtime(CALIBRATE_LIBRARY) >= os.path.getmtime(CALIBRATE_SOURCE)):
+        return CALIBRATE_LIBRARY
+    os.makedirs(GENERATED_DIR, exist_ok=True)
+    cmd = [hipcc_path(), *HIPCC_FLAGS, CALIBRATE_SOURCE, "-o", CALIBRATE_LIBRARY]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise BuildError(f"hipcc failed for the calibration kernel:\n{' '.join(cmd)}\n{proc.stdout}")
+    return CALIBRATE_LIBRARY
+
+
+# ---------------------------------------------------------------------------------------------
 # python -m flexspmv_amd.build --graph NAME [--policy BLOCKxIPT] [-D SWITCH[=VALUE]]... [--out DIR]
 # ---------------------------------------------------------------------------------------------
 VARIANTS_DIR = os.path.join(GENERATED_DIR, "variants")
