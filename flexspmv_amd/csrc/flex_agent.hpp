@@ -48,8 +48,10 @@ template <typename V, int N> __device__ __forceinline__ void zero(Pack<V, N>& a)
   for (int i = 0; i < N; ++i) a.v[i] = V(0);
 }
 
-// Loads of the read-once edge streams and stores of the write-once outputs.  Two tuning switches mark
-// them non-temporal; plain accesses measured faster for both on MI355X.
+// Loads of the read-once edge streams and stores of the write-once outputs.  The stores are
+// non-temporal: neutral on the SpMV workloads (one output value per row), 7 % on the shallow-water kernel
+// (three output arrays, 17 % of its bytes: 44.6 us against 47.9).  Non-temporal loads of the edge streams
+// measured slower (Poisson 256^3: 374 us against 310) and stay a tuning switch.
 #ifdef FLEX_TUNE_NT_LOADS
 template <typename T> __device__ __forceinline__ T stream_load(const T* p) { return __builtin_nontemporal_load(p); }
 #else
@@ -59,10 +61,10 @@ template <typename T> __device__ __forceinline__ T stream_load(const T* p) { ret
 template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) {
   if (v == T(123456789)) *p = v;
 }
-#elif defined(FLEX_TUNE_NT_STORES)
-template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) { __builtin_nontemporal_store(v, p); }
-#else
+#elif defined(FLEX_TUNE_PLAIN_STORES)  // tuning switch
 template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) { *p = v; }
+#else
+template <typename T> __device__ __forceinline__ void stream_store(T* p, T v) { __builtin_nontemporal_store(v, p); }
 #endif
 
 // Merge-path coordinate on diagonal `diag` of the merge of A = row_end[0..num_rows) (end offset of each
