@@ -507,10 +507,6 @@ def test_repeated_calls_with_the_same_arguments_take_the_shortcut_and_stay_check
     smaller[names.index("num_rows")] = w.num_rows - 1
     with pytest.raises(RuntimeError, match="num_rows \\+ 1"):
         ext.merged_spmv_launch(*smaller)
-    del good, bad, smaller, x
-    import gc
-    gc.collect()
-    assert all(r() is None for r in ext._call_state().repeat.tensors) or True   # weak references keep nothing alive
 
 
 def test_row_aligned_selector_preconditions_are_checked():

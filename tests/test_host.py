@@ -225,3 +225,33 @@ def test_matrix_market_workload(tmp_path):
     with pytest.raises(ValueError):
         scipy.io.mmwrite(str(tmp_path / "rect.mtx"), sp.random(5, 7, density=0.5, random_state=2))
         W.matrix_market_spmv(str(tmp_path / "rect.mtx"), fused_dot=True)
+
+
+def test_launcher_keeps_its_previous_arguments_by_weak_reference_only():
+    """The record a launch leaves for the next call with the same arguments must not keep tensors alive."""
+    import gc
+    import weakref
+
+    import torch
+
+    from flexspmv_amd.binding import HipExtension
+
+    class Probe(HipExtension):          # the bookkeeping alone, without a library
+        def __init__(self):
+            import threading
+            self._tls = threading.local()
+            self._param_names = ["vals", "x", "selector_idx", "row_end_offsets", "num_rows", "num_cols"]
+            self._value_names, self._index_names, self._outputs = ["vals", "x"], ["selector_idx"], [None]
+
+    ext = Probe()
+    args = [torch.zeros(5), torch.zeros(4), torch.zeros(5, dtype=torch.int32), torch.zeros(5, dtype=torch.int32), 4, 4]
+    ext._remember(tuple(args), [torch.zeros(4)], 4, 4, 5, "float32", torch.float32, torch.device("cuda", 0), 256)
+    assert ext._same_arguments(tuple(args)) is not None
+    assert ext._same_arguments(tuple(args[:4] + [4, 5])) is None            # another size
+    assert ext._same_arguments(tuple([args[0].clone()] + args[1:])) is None  # another tensor object
+    args[1].resize_(2)
+    assert ext._same_arguments(tuple(args)) is None                          # the same object in another state
+    probe = weakref.ref(args[0])
+    del args
+    gc.collect()
+    assert probe() is None
