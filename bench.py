@@ -5,9 +5,9 @@
 
 A step is one ``merged_spmv_launch`` of the workload's fused sub-graph (all kernels of the launch,
 inputs resident in HBM).  The headline workload is the 3-D 7-point Poisson operator on a 256^3 grid in
-float64: fused ``y = A x`` and ``x . y``; the second target workload, R-MAT scale 22 in float32, is timed in
-the same run and reported under ``other_workloads.rmat`` with its own roofline and CPU baseline.  One JSON
-line is printed:
+float64: fused ``y = A x`` and ``x . y``; the other four workloads (R-MAT scale 22 in float32 - the second
+target workload -, shallow water, spring-mass, 2-D Laplacian) are timed in the same run and reported under
+``other_workloads`` with their own roofline and CPU baseline.  One JSON line is printed:
 
 * ``value``         effective GB/s = algorithmic bytes per step / (wall time of exactly K steps / K)
                     (every streamed array once, every gathered source once, every output once)
@@ -135,7 +135,7 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
     from flexspmv_amd import workloads as W
     from flexspmv_amd.binding import HipExtension, load_named
 
-    ext = HipExtension(library) if library else load_named(w.graph, build_if_missing=False)
+    ext = HipExtension(library, allow_variant=True) if library else load_named(w.graph, build_if_missing=False)
     args = W.launch_arguments(w, ext.param_names(), "cuda:0")
     # Untimed warm-up: W launches, and in any case launches for 60 ms.  Building a workload keeps the host
     # busy for seconds while the GPU idles and clocks down; a handful of sub-millisecond launches is not
@@ -229,6 +229,7 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
     }
     if library:
         result["library"] = library
+        result["library_variant"] = ext.variant   # tuning switches and tile-shape override the file was built with
     if machine:
         result["machine"] = machine
     if ms_per_step_reuse is not None:
@@ -238,41 +239,16 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
     return result, [o.cpu().numpy() for o in outs]
 
 
-FLOOR_ULPS = 8
-
-
-def reducer_row_scales(ir, w, run_oracle, threads):
-    """Per reducer output: (the sum over each row of |what one edge contributes| in float64, the absolute floor
-    FLOOR_ULPS * eps * largest |contribution|): the oracle run on the same edges with every edge as a row of
-    its own (single-term sums, no rounding).  The floor is what two evaluations of a map with a cancellation
-    inside (the spring's r - L) differ by however small the contribution comes out; for products it is far
-    below the row criterion."""
-    import numpy as np
-    ne = int(w.ne)
-    per_edge, _ = run_oracle(ir, w.tensors, np.arange(ne + 1, dtype=np.int32), ne, w.num_cols, threads)
-    starts = np.asarray(w.row_end_offsets[:-1], dtype=np.int64)
-    empty = np.diff(w.row_end_offsets) == 0
-    scales = {}
-    for i, spec in enumerate(ir.outputs):
-        if spec["target"] != "reducer":
-            continue
-        a = np.abs(per_edge[i].astype(np.float64)).reshape(ne, -1)
-        floor = FLOOR_ULPS * float(np.finfo(per_edge[i].dtype).eps) * float(a.max())
-        a = np.vstack([a, np.zeros((1, a.shape[1]))])
-        s = np.add.reduceat(a, np.minimum(starts, ne), axis=0)
-        s[empty] = 0.0
-        scales[i] = (s, floor)
-    return scales
-
-
 def cpu_leg(w, result, outs, cpu_runs):
     """CPU leg, run after every GPU timing is done (its OpenMP threads would otherwise disturb the
-    launch thread): times the oracle on the same inputs and checks the GPU outputs against it."""
+    launch thread): times the oracle on the same inputs and checks the GPU outputs against it with the
+    criterion of oracle/parity.py (row by row; every term of the allowance is the row's own)."""
     import numpy as np
 
     from flexspmv_amd import graphs
     if cpu_runs <= 0:
         return result
+    from oracle.parity import FLOOR_ULPS, MOVE_FACTOR, aggregator_bounds, reducer_row_scales, row_excess
     from oracle.runner import run_oracle
     T = host_threads()
     ir = graphs.get(w.graph)
@@ -286,40 +262,44 @@ def cpu_leg(w, result, outs, cpu_runs):
     times.sort()
     cpu_ms = times[len(times) // 2] * 1e3
     tol = 1e-5 if result["dtype"] == "float32" else 1e-12
-    # Aggregators in float32: the reference sums millions of terms sequentially per thread, so its own
-    # result drifts from the exact sum by far more than the tolerance (and depends on the thread count).
-    # They are therefore checked against the same oracle evaluated in float64; the weaker statement about
-    # the float32 oracle itself (sequential-summation bound) is checked beside it.
-    ref_hi = None
+    scales = reducer_row_scales(ir, w.tensors, w.row_end_offsets, w.num_cols, T) if w.row_end_offsets is not None else {}
+    # worst = the largest |difference| as a multiple of what the criterion allows (<= 1: within the tolerance)
+    worst, fine_ok, aggregators = 0.0, True, {}
     centre = "oracle_" + DTYPE_TAG[result["dtype"]].replace("f", "fp")
-    if result["dtype"] == "float32" and "sum" in result["output_kinds"]:
-        hi = {k: (v.astype(np.float64) if v.dtype == np.float32 else v) for k, v in w.tensors.items()}
-        ref_hi, _ = run_oracle(ir, hi, w.row_end_offsets, w.num_rows, w.num_cols, T)
-        centre = "oracle_fp32 for reducer outputs, oracle_fp64 for aggregator outputs"
-    scales = reducer_row_scales(ir, w, run_oracle, T) if w.row_end_offsets is not None else {}
-    worst, weak_ok = 0.0, True
     for i, (o, r) in enumerate(zip(outs, ref)):
-        o64 = o.astype(np.float64)
-        if ref_hi is not None and result["output_kinds"][i] == "sum":
-            hi_i = ref_hi[i].astype(np.float64)
-            chain = -(-int(w.ne) // T)
-            weak_ok &= bool(np.abs(o64 - r.astype(np.float64)).max()
-                            <= (chain * np.finfo(np.float32).eps + tol) * np.abs(hi_i).max())
-            r64 = hi_i
+        agg = aggregator_bounds(ir, w.tensors, w.row_end_offsets, w.num_rows, w.num_cols, i, tol)
+        if agg is not None:
+            # float32 aggregators: the reference's own sequential float32 sum drifts from the exact sum by far more
+            # than the tolerance, so the centre is the oracle in float64; the distances to the float32 oracle at
+            # this run's thread count and at 256 threads (shortest chains) are reported beside it
+            centre = "oracle_fp32 for reducer outputs, oracle_fp64 for aggregator outputs"
+            o64 = o.astype(np.float64)
+            size = max(float(np.abs(agg["centre"]).max()), 1e-300)
+            to_centre = float(np.abs(o64 - agg["centre"]).max()) / size
+            to_fine = float(np.abs(o64 - agg["fine"].astype(np.float64)).max())
+            fine_ok &= to_fine <= agg["bound_fine"]
+            worst = max(worst, to_centre / tol)
+            aggregators[ir.outputs[i]["name"]] = {
+                "rel_diff_vs_fp64_oracle": to_centre,
+                f"rel_diff_vs_fp32_oracle_{T}_threads": float(np.abs(o64 - r.astype(np.float64)).max()) / size,
+                "rel_diff_vs_fp32_oracle_256_threads": to_fine / size,
+                "bound_vs_fp32_oracle_256_threads": agg["bound_fine"] / size,
+                "fp32_oracle_vs_fp64_oracle": float(np.abs(r.astype(np.float64) - agg["centre"]).max()) / size}
+        elif i in scales:
+            worst = max(worst, float(row_excess(o, r, tol, *scales[i]).max()))
+        elif o.dtype.kind == "i":
+            worst = max(worst, 0.0 if np.array_equal(o, r) else float("inf"))
         else:
             r64 = r.astype(np.float64)
-        if i in scales:
-            row_scale, floor = scales[i]
-            # |diff| <= tol * scale + floor  <=>  |diff| / (scale + floor / tol) <= tol
-            scale = np.maximum(np.abs(r64), row_scale.reshape(r64.shape)) + max(floor / tol, 1e-300)
-            worst = max(worst, float((np.abs(o64 - r64) / scale).max()))
-        else:
-            worst = max(worst, float(np.abs(o64 - r64).max()) / max(float(np.abs(r64).max()), 1e-300))
+            worst = max(worst, float(np.abs(o.astype(np.float64) - r64).max()) / max(float(np.abs(r64).max()), 1e-300) / tol)
     result["cpu"] = {"ms": cpu_ms, "gbs": w.algorithmic_bytes / cpu_ms / 1e6, "threads": T, "runs": cpu_runs,
-                     "max_rel_diff_vs_gpu": worst, "tolerance": tol,
-                     "parity_ok": bool(worst <= tol) and weak_ok, "parity_centre": centre,
-                     "parity_scale": "per row: max(|reference|, sum of |contributions| of the row) + "
-                                     f"{FLOOR_ULPS} ulp of the largest contribution / tolerance; aggregators: |reference|"}
+                     "max_rel_diff_vs_gpu": worst * tol, "tolerance": tol,
+                     "parity_ok": bool(worst <= 1.0) and fine_ok, "parity_centre": centre,
+                     "parity_scale": "per row: max(|reference|, sum of |contributions| of the row); floor per row: "
+                                     f"{FLOOR_ULPS} ulp of the row's largest contribution + {MOVE_FACTOR} x what moves of the "
+                                     "inputs by an ulp or two change in the row's contributions; aggregators: |reference|"}
+    if aggregators:
+        result["cpu"]["float32_aggregators"] = aggregators
     return result
 
 
@@ -346,7 +326,8 @@ def cpu_baseline_of(r):
             "sample": f"the whole workload ({r['workload']}), median of {c['runs']} runs after one warm-up, "
                       f"{c['ms']:.1f} ms per run",
             "ms": c["ms"], "parity_max_rel_diff": c["max_rel_diff_vs_gpu"], "parity_tolerance": c["tolerance"],
-            "parity_ok": c["parity_ok"], "parity_centre": c["parity_centre"], "parity_scale": c["parity_scale"]}
+            "parity_ok": c["parity_ok"], "parity_centre": c["parity_centre"], "parity_scale": c["parity_scale"],
+            **({"float32_aggregators": c["float32_aggregators"]} if "float32_aggregators" in c else {})}
 
 
 def time_edge_list_preparation(w, steps):
@@ -415,7 +396,7 @@ def main() -> int:
     ap.add_argument("--mtx-dot", action="store_true", help="with --mtx: the fused form y = A x and x . y")
     ap.add_argument("--others", default=None,
                     help="comma-separated workloads timed after the headline one and reported under other_workloads "
-                         "(default: rmat when the headline is the default Poisson run; 'none' for none)")
+                         "(default: the other four when the headline is the default Poisson run; 'none' for none)")
     ap.add_argument("--all", action="store_true", help="time all the other four workloads (extra JSON key)")
     ap.add_argument("--cpu-runs", type=int, default=5, help="timed runs of the CPU baseline (0 = skip)")
     ap.add_argument("--no-calibration", action="store_true",
@@ -460,7 +441,8 @@ def main() -> int:
     elif a.others is not None:
         other_names = [n for n in a.others.split(",") if n and n != "none"]
     else:
-        other_names = ["rmat"] if (a.workload == "poisson3d" and a.mtx is None and a.size is None) else []
+        other_names = (["rmat", "shallow_water", "spring_mass", "laplacian2d"]
+                       if (a.workload == "poisson3d" and a.mtx is None and a.size is None) else [])
     pending = []
     for name in other_names:
         wo = W.WORKLOADS[name](DEFAULT_SIZE[name])
@@ -514,6 +496,7 @@ def main() -> int:
         line["config"]["note"] = WORKLOAD_NOTES[a.workload]
     if a.library:
         line["config"]["library"] = a.library   # not the shipped library: a variant built for a measurement
+        line["config"]["library_variant"] = head["library_variant"]
     if "ms_per_step_tile_reuse" in head:
         line["with_tile_reuse"] = {"ms_per_step": head["ms_per_step_tile_reuse"], "value": head["gbs_tile_reuse"],
                                    "unit": "GB/s", "note": "tile table of the previous launch reused "

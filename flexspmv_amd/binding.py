@@ -34,6 +34,7 @@ ABI_VERSION = 4
 FLAG_TIME_KERNEL = 1
 FLAG_REUSE_TILES = 2
 FLAG_KEEP_TILES = 4
+FLAG_DEBUG_SYNC = 8
 DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
 EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
                     "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms", "flexspmv_tiling",
@@ -96,6 +97,14 @@ def load_library(path: str) -> ctypes.CDLL:
     return lib
 
 
+def variant_of(signature: Dict[str, Any]) -> str:
+    """What makes a library a measurement variant - its tuning switches and tile-shape override as text -
+    or "" for a product library."""
+    parts = list(signature.get("tuning", []))
+    parts += [f"{k}={v}" for k, v in sorted(signature.get("policy_override", {}).items())]
+    return " ".join(parts)
+
+
 class _CallState:
     """ctypes objects of one thread's launches of one library (kept alive together)."""
     __slots__ = ("v_arr", "i_arr", "o_arr", "la", "ref", "repeat")
@@ -129,10 +138,16 @@ class HipExtension:
     ``merged_spmv_launch(values..., gathers..., index tensors..., row_end_offsets, num_rows, num_cols)``.
     """
 
-    def __init__(self, lib_path: str) -> None:
+    def __init__(self, lib_path: str, allow_variant: bool = False) -> None:
         self.lib_path = lib_path
         self._lib = load_library(lib_path)
         self.signature: Dict[str, Any] = json.loads(self._lib.flexspmv_signature().decode())
+        # A library built with tuning switches or another tile shape is a measurement variant (some switches
+        # give wrong results on purpose): only a caller that asks for one gets one.
+        self.variant = variant_of(self.signature)
+        if self.variant and not allow_variant:
+            raise RuntimeError(f"{lib_path} is a measurement variant ({self.variant}), not a product library; "
+                               f"pass allow_variant=True to load it for a measurement")
         self._value_names: List[str] = list(self.signature["value_inputs"])
         self._index_names: List[str] = list(self.signature["index_inputs"])
         self._row_aligned = set(self.signature.get("row_aligned_index_inputs", []))
@@ -147,6 +162,8 @@ class HipExtension:
         self._dtypes = set(self.signature["dtypes"])
         self._param_names = [p["name"] for p in self.signature["params"]]
         self._workspace: Dict[Any, Any] = {}   # (device index, stream handle) -> scratch tensor
+        self._last_used: Dict[Any, int] = {}   # ... -> number of the last launch that used it
+        self._launch_count = 0
         self._captured = set()                 # keys whose buffer a stream capture has recorded
         self._retained: List[Any] = []         # replaced buffers that a captured graph still refers to
         self.time_kernel = False   # set True to bracket the dominant kernel of each launch with events
@@ -155,7 +172,8 @@ class HipExtension:
         # Off by default: every launch then does all the work a launch of the reference does.
         self.reuse_tiles = False
         self._tile_key = None
-        self.extra_flags = 0       # FLAG_* bits added to every launch (FLAG_KEEP_TILES for debugging)
+        self.extra_flags = 0       # FLAG_* bits added to every launch (FLAG_DEBUG_SYNC: print every kernel's
+                                   # grid / block / LDS on stderr and synchronize after it)
         # what a launch looks up, prepared once
         self._dispatch_name = self.signature["dispatch_tensor"]
         self._tensor_names = self._value_names + self._index_names + ["row_end_offsets"]
@@ -183,17 +201,24 @@ class HipExtension:
     def workspace_bytes(self, dtype: str, num_rows: int, ne: int) -> int:
         return int(self._lib.flexspmv_workspace_bytes(DTYPE_CODES[dtype], num_rows, ne))
 
+    # scratch buffers kept at most, before those of streams that have not launched for a while are dropped
+    MAX_IDLE_SCRATCH = 8
+    IDLE_LAUNCHES = 64
+
     def _scratch(self, device, index: int, raw_stream: int, nbytes: int):
         """Scratch of this library for launches on the stream with handle ``raw_stream`` of device ``index``
         (the current stream of the current device when this is called).
 
         The buffer is allocated on that stream and only ever used on it, so when a larger launch replaces
-        it the caching allocator hands the old block out again in stream order - nothing still running
-        can see it change.  A buffer that a stream capture has recorded is kept for the life of the
-        library (a replayed graph keeps using its address), and growing during a capture is refused:
-        run the step once eagerly first, as capture_step does."""
+        it - or when it is dropped - the caching allocator hands the old block out again in stream order:
+        nothing still running can see it change.  A buffer that a stream capture has recorded is kept for
+        the life of the library (a replayed graph keeps using its address), and growing during a capture
+        is refused: run the step once eagerly first, as capture_step does.  A caller that cycles through
+        many streams does not grow the table without bound: beyond MAX_IDLE_SCRATCH entries, buffers of
+        streams that have not launched for IDLE_LAUNCHES launches are dropped (never a captured one)."""
         import torch
         key = (index, raw_stream)
+        self._launch_count += 1
         buf = self._workspace.get(key)
         capturing = torch._C._cuda_isCurrentStreamCapturing()
         if buf is None or buf.numel() < nbytes:
@@ -204,9 +229,23 @@ class HipExtension:
                 self._captured.discard(key)
             buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
             self._workspace[key] = buf
+            if len(self._workspace) > self.MAX_IDLE_SCRATCH:
+                self._drop_idle_scratch(key)
+        self._last_used[key] = self._launch_count
         if capturing:
             self._captured.add(key)
         return buf
+
+    def _drop_idle_scratch(self, keep) -> None:
+        for k in list(self._workspace):
+            if k != keep and k not in self._captured and \
+                    self._launch_count - self._last_used.get(k, 0) >= self.IDLE_LAUNCHES:
+                # a tile table remembered in the dropped buffer is gone with it (the block may come back at
+                # the same address with other contents)
+                if self._tile_key is not None and self._tile_key[5] == self._workspace[k].data_ptr():
+                    self._tile_key = None
+                del self._workspace[k]
+                self._last_used.pop(k, None)
 
     def workspace_of(self, device, stream=None):
         """The scratch tensor of launches on ``stream`` (default: the current stream) of ``device``, or
@@ -244,8 +283,8 @@ class HipExtension:
 
     def _same_arguments(self, args):
         """The record of the previous call on this thread if ``args`` are the same objects in the same state
-        (same tensors - weak references, so nothing is kept alive -, same storage, size and layout; equal
-        sizes), else None."""
+        (same tensors - weak references, so nothing is kept alive -, same storage, size, dtype, device and
+        layout; equal sizes), else None."""
         st = getattr(self._tls, "state", None)
         rep = st.repeat if st is not None else None
         if rep is None or len(args) != len(rep.args):
@@ -256,9 +295,10 @@ class HipExtension:
                     return None
             elif a.__class__ is not known.__class__ or a != known:
                 return None
-        for t, (ptr, count) in zip(rep.tensors, rep.state):
+        for t, (ptr, count, dtype, device) in zip(rep.tensors, rep.state):
             t = t()
-            if t.data_ptr() != ptr or t.numel() != count or not t.is_contiguous():
+            if (t.data_ptr() != ptr or t.numel() != count or t.dtype != dtype or t.device != device
+                    or not t.is_contiguous()):
                 return None
         return rep
 
@@ -369,7 +409,7 @@ class HipExtension:
             rep.tensors = tuple(weakref.ref(t) for t in tensors)
         except TypeError:      # an argument type that cannot be weakly referenced: no shortcut
             return
-        rep.state = tuple((t.data_ptr(), t.numel()) for t in tensors)
+        rep.state = tuple((t.data_ptr(), t.numel(), t.dtype, t.device) for t in tensors)
         where = {n: i for i, n in enumerate(self._param_names)}
         rep.value_pos = tuple(where[n] for n in self._value_names)
         rep.index_pos = tuple(where[n] for n in self._index_names)

@@ -66,10 +66,11 @@ def graph_dir(ir: FusedGraphIR, out_dir: Optional[str] = None) -> str:
 
 def write_generated_source(ir: FusedGraphIR, out_dir: Optional[str] = None,
                            dtypes: Optional[Sequence[str]] = None,
-                           policy: Optional[Dict[str, int]] = None) -> Tuple[str, Dict[str, Any]]:
+                           policy: Optional[Dict[str, int]] = None,
+                           defines: Sequence[str] = ()) -> Tuple[str, Dict[str, Any]]:
     """Emit ``<name>.hip`` for a sub-graph; returns (path, signature)."""
     from .codegen.merged_gen_gpu import generate_hip_source
-    src, signature = generate_hip_source(ir, dtypes=dtypes, policy=policy)
+    src, signature = generate_hip_source(ir, dtypes=dtypes, policy=policy, defines=defines)
     d = graph_dir(ir, out_dir)
     os.makedirs(d, exist_ok=True)
     path = os.path.join(d, f"{ir.name}.hip")
@@ -108,8 +109,10 @@ def is_current(ir: FusedGraphIR, out_dir: Optional[str] = None) -> bool:
 def compile_graph(ir: FusedGraphIR, out_dir: Optional[str] = None, force: bool = False,
                   dtypes: Optional[Sequence[str]] = None, policy: Optional[Dict[str, int]] = None,
                   extra_flags: Sequence[str] = ()) -> str:
-    """Generate + compile; returns the path of the shared library."""
-    src, _ = write_generated_source(ir, out_dir, dtypes=dtypes, policy=policy)
+    """Generate + compile; returns the path of the shared library.  ``-DFLEX_TUNE_*`` entries of
+    ``extra_flags`` are tuning switches: the generator records them in the library's signature."""
+    defines = [f[2:] for f in extra_flags if f.startswith("-DFLEX_TUNE_")]
+    src, _ = write_generated_source(ir, out_dir, dtypes=dtypes, policy=policy, defines=defines)
     lib = library_path(ir, out_dir)
     if not force and is_current(ir, out_dir):
         return lib

@@ -218,12 +218,16 @@ def _choose_ipt(kp: KernelPlan, value_bytes: int) -> int:
 
 
 def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None,
-                        policy: Optional[Dict[str, int]] = None) -> Tuple[str, Dict[str, Any]]:
+                        policy: Optional[Dict[str, int]] = None,
+                        defines: Sequence[str] = ()) -> Tuple[str, Dict[str, Any]]:
     """Return (translation unit text, signature dict) for a sub-graph.
 
     ``dtypes`` lists the value types to instantiate (default float32 + float64, plus int64 when the
     dispatch input was traced as int64 - the reference's rule, codegen/merged_gen_binding.py:143-157).
     ``policy`` may override ``block``, ``ipt_f32``, ``ipt_f64`` and ``ipt_flat``.
+    ``defines`` are the ``FLEX_TUNE_*`` switches (``NAME`` or ``NAME=VALUE``) the library will be compiled
+    with.  A library with a policy override or switches is a measurement variant: both are recorded in the
+    signature (``"tuning"``, ``"policy_override"``), and loaders of product libraries refuse it.
     """
     inputs, outputs, selector_register, map_ops, red_ops, agg_ops = ir.six()
     kp = analyse(ir)
@@ -233,6 +237,10 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         dtypes = ["float32", "float64"] + (["int64"] if plan.allow_int64 else [])
     dtypes = [dtype_name(d) for d in dtypes]
     policy = dict(policy or {})
+    defines = sorted(str(d) for d in defines)
+    for d in defines:
+        if not d.startswith("FLEX_TUNE_"):
+            raise ValueError(f"{d!r} is not a tuning switch (FLEX_TUNE_*)")
     block = int(policy.get("block", BLOCK_THREADS))
     ipt = {"float32": int(policy.get("ipt_f32", _choose_ipt(kp, 4))),
            "float64": int(policy.get("ipt_f64", _choose_ipt(kp, 8))),
@@ -343,6 +351,9 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         # value tensors read at index `row` for every row of a tile: they must hold at least num_rows items
         "row_indexed_value_inputs": sorted({src for _, src, _, _ in kp.row_sources}),
         "policy": {"block": block, "ipt": {k: ipt[k] for k in dtypes}},
+        # what makes this library a measurement variant instead of a product library (both empty: product)
+        "policy_override": {k: int(v) for k, v in sorted(policy.items())},
+        "tuning": defines,
         "widths": {"fetch_values": kp.fetch_value_width, "fetch_indices": kp.fetch_index_width,
                    "reduce": kp.red_width, "aggregate": kp.agg_width, "row": kp.row_width},
     })
@@ -363,6 +374,7 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
 
     src = f"""// Generated by flexspmv_amd.codegen.merged_gen_gpu for sub-graph "{ir.name}" ({ir.content_hash()}).
 // Do not edit: regenerate from the six-list description instead.
+#define FLEX_TUNING_DECLARED {1 if defines else 0}  // tuning switches given to the generator: {" ".join(defines) or "none"}
 #include "flex_dispatch.hpp"
 
 namespace {{

@@ -33,12 +33,22 @@
 
 #include <type_traits>
 
+#include "flex_tuning.hpp"
 #include "flex_tensor.hpp"
 #include "flex_wave.hpp"
 
 namespace flex {
 
 constexpr int NUM_XCD = 8;
+
+// Aggregator partials a reducer block leaves per tile: one (its wavefronts' partials are added in the block,
+// in wavefront order).  One per wavefront - no barrier at the end of the block, four times the words for
+// the fix-up to read - measured 2 - 3 us slower per launch on Poisson 256^3 (step 319.2 us against 316.9).
+#ifdef FLEX_TUNE_PARTIAL_PER_WAVE
+template <int BLOCK> constexpr int partials_per_tile() { return BLOCK / 64; }
+#else
+template <int BLOCK> constexpr int partials_per_tile() { return 1; }
+#endif
 
 
 template <typename V, int N> struct Pack { V v[N > 0 ? N : 1]; };
@@ -843,13 +853,31 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
     }
   }
 
-  // one aggregator partial per wavefront of the tile (fixup_kernel adds them in a fixed order)
+  // one aggregator partial per tile: the wavefronts' partials added in wavefront order (fixup_kernel adds the
+  // tiles' partials in a fixed order)
   if constexpr (AGG > 0) {
     wave_sum_to_last_lane<V, AGG>(agg.v);
+#ifndef FLEX_TUNE_PARTIAL_PER_WAVE
+    __shared__ V s_tile_agg[NW][AGG];
+    if (lane == WAVE - 1) {
+#pragma unroll
+      for (int c = 0; c < AGG; ++c) s_tile_agg[wave][c] = agg.v[c];
+    }
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+      for (int c = 0; c < AGG; ++c) {
+        V t = s_tile_agg[0][c];
+        for (int w = 1; w < NW; ++w) t += s_tile_agg[w][c];
+        agg_partials[(size_t)tile * AGG + c] = t;
+      }
+    }
+#else  // tuning switch: one partial per wavefront, no barrier
     if (lane == WAVE - 1) {
 #pragma unroll
       for (int c = 0; c < AGG; ++c) agg_partials[((size_t)tile * NW + wave) * AGG + c] = agg.v[c];
     }
+#endif
   }
 }
 
@@ -867,8 +895,11 @@ __global__ void __launch_bounds__(BLOCK)
 reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_rows, const int* __restrict__ row_end,
               const int nnz, const typename G::Params p, int* __restrict__ carry_row,
               typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials,
-              int2* __restrict__ coords_out) {
+              int2* __restrict__ coords_out, unsigned* __restrict__ ticket) {
   const int num_tiles = tl.num_tiles;
+#ifdef FLEX_TUNE_TICKET_SUM
+  if (blockIdx.x == 0 && threadIdx.x == 0) *ticket = 0u;  // arms the last-block detection of fixup_kernel
+#endif
 #ifdef FLEX_TUNE_PERSISTENT
   int tile = blockIdx.x;
   if (tile >= num_tiles) return;
@@ -994,20 +1025,21 @@ flat_kernel(const typename G::Params p, const int nnz, const int num_tiles,
 // tiles BLOCK at a time for as long as they carry into that row and adds them up in a fixed order; the
 // chunks those tiles belong to see that their leading tiles continue an earlier run and leave them alone.
 // Nothing here depends on timing: the same sums in the same order on every run, no atomics.
-// The aggregator partials (PARTS_PER_TILE per tile, one per wavefront of the reducer block) are summed in a
+// The aggregator partials (PARTS_PER_TILE per tile: one, or one per wavefront of the reducer block) are summed in a
 // fixed order.
 //   SINGLE = false: block b handles tiles [b*BLOCK, (b+1)*BLOCK) and leaves its aggregator sum in
 //                   block_partials[b]; aggregate_kernel adds those, again in a fixed order.
 //   SINGLE = true:  one block walks all chunks (launches of a few thousand tiles) and assigns the
 //                   aggregator outputs itself: one kernel less.
-// (Finishing the sum in the last fix-up block to finish, found with a ticket counter, was measured and
-// is slower: the release fence each block needs writes the XCD's whole L2 back, output rows included.)
+// (Finishing the sum in the last fix-up block to finish, found with a ticket counter - FLEX_TUNE_TICKET_SUM -,
+// was measured twice and is slower, also with the row outputs stored non-temporally: Poisson 256^3 step
+// 323.0 us against 319.0; each block's release at device scope costs more than the 4.6 us kernel it saves.)
 // ----------------------------------------------------------------------------------------------
 template <class G, int BLOCK, int PARTS_PER_TILE, bool SINGLE>
 __global__ void __launch_bounds__(BLOCK)
 fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restrict__ carry_row,
              const typename G::Value* __restrict__ carry_val, const typename G::Value* __restrict__ agg_partials,
-             typename G::Value* __restrict__ block_partials) {
+             typename G::Value* __restrict__ block_partials, unsigned* __restrict__ ticket) {
   using V = typename G::Value;
   constexpr int RED = G::RED_WIDTH, AGG = G::AGG_WIDTH;
   constexpr int REDN = RED > 0 ? RED : 1;
@@ -1193,6 +1225,8 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
   }
   if constexpr (AGG > 0) {
     __shared__ V s_wave_agg[NW][AGG];
+    __shared__ int s_is_last;
+    (void)s_is_last;
     wave_sum_to_last_lane<V, AGG>(acc.v);
     if (lane == WAVE - 1) {
 #pragma unroll
@@ -1210,10 +1244,55 @@ fixup_kernel(const typename G::Params p, const int num_tiles, const int* __restr
       if constexpr (SINGLE) {
         G::store_agg(p, total);
       } else {
+#ifdef FLEX_TUNE_TICKET_SUM
+        // tuning switch (measured slower, see fixup_kernel's header): the block that draws the last ticket adds the
+        // blocks' partials itself.  Each block publishes its partial before it takes a ticket (release at device
+        // scope), the last one acquires after taking its own.  The reducer kernel zeroes the ticket.
+#pragma unroll
+        for (int c = 0; c < AGG; ++c)
+          __hip_atomic_store(&block_partials[(size_t)blockIdx.x * AGG + c], total.v[c], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+        __atomic_thread_fence(__ATOMIC_RELEASE);
+        const unsigned drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        s_is_last = (drawn == gridDim.x - 1) ? 1 : 0;
+#else
 #pragma unroll
         for (int c = 0; c < AGG; ++c) block_partials[(size_t)blockIdx.x * AGG + c] = total.v[c];
+#endif
       }
     }
+#ifdef FLEX_TUNE_TICKET_SUM
+    if constexpr (!SINGLE) {
+      __syncthreads();
+      if (s_is_last) {
+        __atomic_thread_fence(__ATOMIC_ACQUIRE);
+        Pack<V, AGG> fin;
+        zero(fin);
+        for (int j = tid; j < (int)gridDim.x; j += BLOCK) {
+#pragma unroll
+          for (int c = 0; c < AGG; ++c)
+            fin.v[c] += __hip_atomic_load(&block_partials[(size_t)j * AGG + c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        wave_sum_to_last_lane<V, AGG>(fin.v);
+        __syncthreads();
+        if (lane == WAVE - 1) {
+#pragma unroll
+          for (int c = 0; c < AGG; ++c) s_wave_agg[wave][c] = fin.v[c];
+        }
+        __syncthreads();
+        if (tid == 0) {
+          Pack<V, AGG> total;
+#pragma unroll
+          for (int c = 0; c < AGG; ++c) {
+            V t = s_wave_agg[0][c];
+            for (int w = 1; w < NW; ++w) t += s_wave_agg[w][c];
+            total.v[c] = t;
+          }
+          G::store_agg(p, total);
+        }
+      }
+    }
+#endif
   }
 }
 

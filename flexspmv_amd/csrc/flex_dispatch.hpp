@@ -11,6 +11,7 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include <mutex>
 
@@ -20,8 +21,9 @@
 // Scratch of flexspmv_launch_static: device memory that belongs to the library itself, so that entry point
 // never allocates.  One copy exists on every GPU the library is loaded on, at its own address; host code
 // reaches it only through the per-device pointer that static_scratch() resolves (the array's name is
-// a host-side stand-in, not a device address).
-static __device__ __align__(256) unsigned char scratch[FLEXSPMV_STATIC_SCRATCH_BYTES];
+// a host-side stand-in, not a device address).  File scope, internal linkage, and a name no generated
+// identifier can take (those start with q_ or carry a graph's tensor names inside Graph<>).
+static __device__ __align__(256) unsigned char flexspmv_static_scratch_bytes[FLEXSPMV_STATIC_SCRATCH_BYTES];
 
 namespace flex {
 
@@ -56,7 +58,7 @@ inline int last_kernel_ms(float* ms) {
   return FLEXSPMV_OK;
 }
 
-// Address of `scratch` on the current device, resolved once per device (the first call on a device asks
+// Address of flexspmv_static_scratch_bytes on the current device, resolved once per device (the first call on a device asks
 // the runtime; later calls read the table).  NULL with g_last_error set when the runtime refuses.
 constexpr int MAX_DEVICES = 64;
 inline char* static_scratch() {
@@ -75,14 +77,41 @@ inline char* static_scratch() {
   std::lock_guard<std::mutex> guard(lock);
   if (table[device] == nullptr) {
     void* ptr = nullptr;
-    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(flexspmv_static_scratch_bytes));
     if (e != hipSuccess || ptr == nullptr) {
-      fail_hip(e, "hipGetSymbolAddress(scratch)");
+      fail_hip(e, "hipGetSymbolAddress(flexspmv_static_scratch_bytes)");
       return nullptr;
     }
     table[device] = ptr;
   }
   return (char*)table[device];
+}
+
+// Launch-shape printing, the reference's debug_synchronous (cuda_template/reducer/merged_spmv_template.cuh:106-124,
+// :131-137): with FLEXSPMV_FLAG_DEBUG_SYNC in args->flags, or FLEXSPMV_DEBUG_LAUNCH=1 in the environment, every
+// kernel of a launch is reported on stderr - grid, block, static LDS bytes, registers - and the stream is
+// synchronized after it so that an error names its kernel (no synchronization while the stream is being captured).
+inline bool debug_launch_env() {
+  static const bool on = [] {
+    const char* v = getenv("FLEXSPMV_DEBUG_LAUNCH");
+    return v != nullptr && v[0] != 0 && v[0] != '0';
+  }();
+  return on;
+}
+template <typename KernelT>
+inline int debug_report(const char* name, KernelT kernel, unsigned grid, unsigned block, hipStream_t stream) {
+  hipFuncAttributes attr{};
+  const bool known = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(kernel)) == hipSuccess;
+  fprintf(stderr, "[flexspmv] %s<<<%u, %u, 0, %p>>>  static LDS %zu B, %d registers per thread\n", name, grid, block,
+          (void*)stream, known ? attr.sharedSizeBytes : (size_t)0, known ? attr.numRegs : 0);
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return FLEXSPMV_OK;
+  }
+  const hipError_t e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) return fail_hip(e, name);
+  return FLEXSPMV_OK;
 }
 
 constexpr size_t align_up(size_t n, size_t a = 256) { return (n + a - 1) / a * a; }
@@ -142,7 +171,7 @@ struct Dispatch {
     int carry_blocks;
     bool search_in_blocks;
     bool single_fixup;
-    size_t off_coords, off_carry_row, off_carry_val, off_partials, off_block_partials, total;
+    size_t off_coords, off_carry_row, off_carry_val, off_partials, off_block_partials, off_ticket, total;
   };
 
   // Row-snapped tiles pay with smaller tiles (capacity minus the slack a boundary may be moved by), so
@@ -199,10 +228,14 @@ struct Dispatch {
     if (REDUCER) off += align_up(sizeof(V) * (size_t)l.num_tiles * (G::RED_WIDTH > 0 ? G::RED_WIDTH : 1));
     l.carry_blocks = (l.num_tiles + FIXUP_BLOCK - 1) / FIXUP_BLOCK;
     l.off_partials = off;
-    const size_t parts = REDUCER ? (size_t)l.num_tiles * (BLOCK / WAVE) : (size_t)MAX_PERSISTENT_BLOCKS;
+    const size_t parts = REDUCER ? (size_t)l.num_tiles * partials_per_tile<BLOCK>() : (size_t)MAX_PERSISTENT_BLOCKS;
     if (G::AGG_WIDTH > 0) off += align_up(sizeof(V) * parts * G::AGG_WIDTH);
     l.off_block_partials = off;
     if (REDUCER && G::AGG_WIDTH > 0) off += align_up(sizeof(V) * (size_t)l.carry_blocks * G::AGG_WIDTH);
+    l.off_ticket = off;
+#ifdef FLEX_TUNE_TICKET_SUM
+    off += align_up(sizeof(unsigned));
+#endif
     l.total = off;
     return true;
   }
@@ -273,6 +306,11 @@ struct Dispatch {
     hipStream_t stream = (hipStream_t)a->stream;
     const bool timed = (a->flags & FLEXSPMV_FLAG_TIME_KERNEL) != 0 && g_timer.ready();
     if (timed) g_timer.armed = false;  // untimed launches leave the last timed kernel's events readable
+    const bool debug = (a->flags & FLEXSPMV_FLAG_DEBUG_SYNC) != 0 || debug_launch_env();
+    int debug_rc = FLEXSPMV_OK;
+    auto report = [&](const char* name, auto kernel, int grid, int block) {
+      if (debug && debug_rc == FLEXSPMV_OK) debug_rc = debug_report(name, kernel, (unsigned)grid, (unsigned)block, stream);
+    };
     V* partials = (V*)(ws + l.off_partials);
     const int nnz = (int)a->ne;
 
@@ -282,12 +320,17 @@ struct Dispatch {
       int2* coords = (int2*)(ws + l.off_coords);
       int* carry_row = (int*)(ws + l.off_carry_row);
       V* carry_val = (V*)(ws + l.off_carry_val);
+      unsigned* ticket = (unsigned*)(ws + l.off_ticket);
+      if (debug)
+        fprintf(stderr, "[flexspmv] reducer launch: %d rows, %d non-zeros, %d tiles of %d merge items (capacity %d, snap slack %d), "
+                "%zu bytes of scratch\n", num_rows, nnz, l.num_tiles, l.tiling.nominal, TILE, l.tiling.snap_slack, l.total);
 
       if (!l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0) {
         constexpr int per_block = SEARCH_BLOCK / SEARCH_GROUP;
         const int search_blocks = (l.num_tiles + 1 + per_block - 1) / per_block;
         hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(SEARCH_BLOCK), 0, stream, l.tiling, row_end,
                            num_rows, nnz, coords);
+        report("tile_search_kernel", tile_search_kernel, search_blocks, SEARCH_BLOCK);
       }
 #ifdef FLEX_TUNE_PERSISTENT
       const int reduce_grid = l.num_tiles < 256 * FLEX_TUNE_PERSISTENT ? l.num_tiles : 256 * FLEX_TUNE_PERSISTENT;
@@ -302,35 +345,45 @@ struct Dispatch {
       // launches with short regular rows (row-snapped tiles) take several neighbouring edges per load
       constexpr int EPL = edges_per_load<G, IPT>();
       const bool wide_loads = EPL > 1 && l.tiling.snap_slack > 0 && nnz >= EPL;
-      auto launch_reducer = [&](auto kernel) {
+      auto launch_reducer = [&](auto kernel, const char* name) {
         if (timed) {
           hipExtLaunchKernelGGL(kernel, dim3(reduce_grid), dim3(BLOCK), 0, stream, g_timer.start, g_timer.stop, 0, table,
-                                l.tiling, num_rows, row_end, nnz, p, carry_row, carry_val, partials, table_out);
+                                l.tiling, num_rows, row_end, nnz, p, carry_row, carry_val, partials, table_out, ticket);
           g_timer.armed = true;
         } else {
           hipLaunchKernelGGL(kernel, dim3(reduce_grid), dim3(BLOCK), 0, stream, table, l.tiling, num_rows, row_end, nnz, p,
-                             carry_row, carry_val, partials, table_out);
+                             carry_row, carry_val, partials, table_out, ticket);
         }
+        report(name, kernel, reduce_grid, BLOCK);
       };
-      if (wide_loads) launch_reducer(reduce_kernel<G, BLOCK, IPT, EPL>);
-      else launch_reducer(reduce_kernel<G, BLOCK, IPT, 1>);
+      if (wide_loads) launch_reducer(reduce_kernel<G, BLOCK, IPT, EPL>, "reduce_kernel (several edges per load)");
+      else launch_reducer(reduce_kernel<G, BLOCK, IPT, 1>, "reduce_kernel");
       V* block_partials = (V*)(ws + l.off_block_partials);
+      constexpr int PARTS = partials_per_tile<BLOCK>();
       if (l.single_fixup) {
-        hipLaunchKernelGGL((fixup_kernel<G, SINGLE_FIXUP_BLOCK, BLOCK / WAVE, true>), dim3(1), dim3(SINGLE_FIXUP_BLOCK), 0,
+        hipLaunchKernelGGL((fixup_kernel<G, SINGLE_FIXUP_BLOCK, PARTS, true>), dim3(1), dim3(SINGLE_FIXUP_BLOCK), 0,
                            stream, p, l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials,
-                           block_partials);
+                           block_partials, ticket);
+        report("fixup_kernel (one block)", fixup_kernel<G, SINGLE_FIXUP_BLOCK, PARTS, true>, 1, SINGLE_FIXUP_BLOCK);
       } else {
-        hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, BLOCK / WAVE, false>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0,
+        hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, PARTS, false>), dim3(l.carry_blocks), dim3(FIXUP_BLOCK), 0,
                            stream, p, l.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials,
-                           block_partials);
+                           block_partials, ticket);
+        report("fixup_kernel", fixup_kernel<G, FIXUP_BLOCK, PARTS, false>, l.carry_blocks, FIXUP_BLOCK);
+#ifndef FLEX_TUNE_TICKET_SUM
         if (G::AGG_WIDTH > 0) {
           hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
                              (const V*)block_partials, l.carry_blocks);
+          report("aggregate_kernel", aggregate_kernel<G, FIXUP_BLOCK>, 1, FIXUP_BLOCK);
         }
+#endif
       }
     } else {
       int grid = resident_grid(flat_kernel<G, BLOCK, IPT>, BLOCK, grid_cache);
       if (grid > l.num_tiles) grid = l.num_tiles;
+      if (debug)
+        fprintf(stderr, "[flexspmv] flat launch: %d edges, %d tiles of %d edges, %zu bytes of scratch\n", nnz, l.num_tiles,
+                TILE, l.total);
       if (timed) {
         hipExtLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream, g_timer.start,
                               g_timer.stop, 0, p, nnz, l.num_tiles, partials);
@@ -339,14 +392,16 @@ struct Dispatch {
         hipLaunchKernelGGL((flat_kernel<G, BLOCK, IPT>), dim3(grid), dim3(BLOCK), 0, stream, p, nnz, l.num_tiles,
                            partials);
       }
+      report("flat_kernel", flat_kernel<G, BLOCK, IPT>, grid, BLOCK);
       if (G::AGG_WIDTH > 0) {
         hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p,
                            (const V*)partials, grid);
+        report("aggregate_kernel", aggregate_kernel<G, FIXUP_BLOCK>, 1, FIXUP_BLOCK);
       }
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail_hip(e, "kernel launch failed");
-    return FLEXSPMV_OK;
+    return debug_rc;
   }
 };
 
@@ -354,7 +409,8 @@ inline int check_counts(const flexspmv_launch_args* a, int nv, int ni, int no) {
   if (a == nullptr) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "args is NULL");
   if (a->struct_size != sizeof(flexspmv_launch_args))
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "struct_size does not match this library's flexspmv_launch_args");
-  if ((a->flags & ~(FLEXSPMV_FLAG_TIME_KERNEL | FLEXSPMV_FLAG_REUSE_TILES | FLEXSPMV_FLAG_KEEP_TILES)) != 0)
+  if ((a->flags & ~(FLEXSPMV_FLAG_TIME_KERNEL | FLEXSPMV_FLAG_REUSE_TILES | FLEXSPMV_FLAG_KEEP_TILES |
+                    FLEXSPMV_FLAG_DEBUG_SYNC)) != 0)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "unknown bits in flags");
   if (a->num_value_inputs != nv || a->num_index_inputs != ni || a->num_outputs != no)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "argument counts do not match flexspmv_signature()");

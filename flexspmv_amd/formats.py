@@ -128,6 +128,19 @@ def sort_edges_by_row(row_ids, num_rows: int) -> Tuple["torch.Tensor", "torch.Te
     return sorted_rows, permutation
 
 
+def mark_written(t) -> None:
+    """Tell torch that ``t`` was written through its raw pointer (a kernel of this package, not a torch
+    operation): the tensor's version counter goes up, as it does for torch's own in-place operations, so
+    that whoever keys a cache on it (autograd's saved-tensor check, the wrapper's copies of unchanged edge
+    tensors) sees the change."""
+    import torch
+    bump = getattr(torch.autograd.graph, "increment_version", None)
+    if bump is not None:
+        bump(t)
+    else:                      # older torch: an in-place no-op on an empty slice bumps the counter too
+        t[:0].zero_()
+
+
 def _permute(fn_name: str, src, permutation, out=None):
     import torch
     if not (src.is_cuda and permutation.is_cuda):
@@ -141,6 +154,7 @@ def _permute(fn_name: str, src, permutation, out=None):
     row_bytes = (src.numel() // max(n, 1)) * src.element_size()
     if n and row_bytes % 4 != 0:
         raise RuntimeError("one entry of the tensor must be a multiple of 4 bytes")
+    given = out is not None
     if out is None:
         out = torch.empty_like(src)
     elif not (out.is_contiguous() and out.shape == src.shape and out.dtype == src.dtype and out.device == src.device):
@@ -148,6 +162,8 @@ def _permute(fn_name: str, src, permutation, out=None):
     with torch.cuda.device(src.device):
         _check(getattr(library(), fn_name)(src.data_ptr(), out.data_ptr(), permutation.contiguous().data_ptr(), n,
                                            row_bytes, _stream(src)))
+    if given:
+        mark_written(out)      # the caller's tensor changed behind torch's back
     return out
 
 

@@ -169,6 +169,40 @@ def bpoints_copy(dtype="int64") -> FusedGraphIR:
     return b.build()
 
 
+def index_spmv(dtype="int64") -> FusedGraphIR:
+    """Integer SpMV with a total: ``y = reducer(w * selector(ids))`` and ``sum(w * selector(ids))`` on int64
+    data, the value type the reference dispatches for sub-graphs traced on int64 tensors
+    (codegen/merged_gen_binding.py:143-157).  Integer sums have one right answer whatever the order, so
+    this sub-graph holds the reducer, the carry fix-up and the aggregator to bit-exactness."""
+    b = GraphBuilder("index_spmv", dtype, doc=index_spmv.__doc__)
+    b.placeholder("w", (1,))
+    b.placeholder("ids", (1,))
+    b.select("selector", "ids")
+    b.map("mul", "mul", ["w", "selector"])
+    b.reduce("reducer", "mul")
+    b.aggregate("sum_1", "mul")
+    b.output("reducer", "sum_1")
+    return b.build()
+
+
+def index_sums(dtype="int64") -> FusedGraphIR:
+    """Integer sub-graph with a row-aligned source, two reducers of widths 2 and 1 on one row structure
+    and an aggregator of width 2, on int64 data (mesh bookkeeping such as per-cell sums of neighbour ids
+    and weighted degrees; assemble_shallow_water.py:62-77 shuffles indices the same way)."""
+    b = GraphBuilder("index_sums", dtype, doc=index_sums.__doc__)
+    b.placeholder("w", (1,))
+    b.placeholder("ids", (2,))
+    b.select("sel", "ids")
+    b.select("sel_row", "ids", row_aligned=True)
+    b.map("mul", "mul", ["sel", "w"], shape=(2,))
+    b.map("sub", "sub", ["mul", "sel_row"])
+    b.reduce("red", "sub")
+    b.reduce("weight", "w", module="red")
+    b.aggregate("sum_1", "mul")
+    b.output("red", "weight", "sum_1")
+    return b.build()
+
+
 def op_zoo(dtype="float32") -> FusedGraphIR:
     """Every element-wise op of the reference's emitters in one reducer sub-graph, including the
     corner cases of the value type: guarded and unguarded division, modulo broadcast between widths
@@ -244,6 +278,8 @@ REGISTRY: Dict[str, Callable[..., FusedGraphIR]] = {
     "mass_sum": mass_sum,
     "system_two_selectors": system_two_selectors,
     "bpoints_copy": bpoints_copy,
+    "index_spmv": index_spmv,
+    "index_sums": index_sums,
     "op_zoo": op_zoo,
     "map_store": map_store,
 }

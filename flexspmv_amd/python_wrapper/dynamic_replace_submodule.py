@@ -27,6 +27,7 @@ import torch
 import torch.nn as nn
 
 from .. import formats as _formats
+from ..formats import mark_written as _mark_written
 from ..frontend.lite import Reducer, Selector
 from .edge_order import gather_edges, scatter_edges, stable_sort_by_row
 
@@ -232,10 +233,14 @@ class _DynamicCudaWrapper(nn.Module):
         call_args += [ro, num_rows, num_cols]
 
         outs = self._ext.merged_spmv_launch(*call_args)
-        if perm is not None:            # per-edge stores went to the sorted copies: put them back
-            for n, a in zip(self._input_param_names, args):
-                if n in self._written_inputs and n in self._non_gather_value_inputs:
-                    scatter_edges(arg_map[n], perm, out=a)
+        # The kernel stored into the written inputs through raw pointers: their version counters go up as they
+        # would after torch's own in-place operations, so that nobody (this class's copies of unchanged edge
+        # tensors in another wrapper included) mistakes them for unchanged.
+        for n, a in zip(self._input_param_names, args):
+            if n in self._written_inputs:
+                if perm is not None and n in self._non_gather_value_inputs:
+                    scatter_edges(arg_map[n], perm, out=a)      # stores went to the sorted copy: put them back
+                _mark_written(a)
         if outs is None:
             return []
         outs = list(outs) if isinstance(outs, (tuple, list)) else [outs]

@@ -53,6 +53,12 @@ extern "C" {
  * a CPU merge-path search (see flexspmv_tiling for the diagonals).  This flag is accepted and changes
  * nothing (it used to ask small launches for the table). */
 #define FLEXSPMV_FLAG_KEEP_TILES 4u
+/* The reference's debug_synchronous argument (cuda_template/reducer/merged_spmv_template.cuh:106-124,131-137):
+ * every kernel of the launch is reported on stderr (grid, block, static LDS bytes, registers) and the stream is
+ * synchronized after it, so that an error is returned by the launch that caused it and names its kernel.  The
+ * environment variable FLEXSPMV_DEBUG_LAUNCH=1 turns the same on for every launch of the process.  While the
+ * stream is being captured the report is printed and the synchronization left out. */
+#define FLEXSPMV_FLAG_DEBUG_SYNC 8u
 
 /* Value types a library may have been generated for (flexspmv_launch_args.dtype). */
 enum flexspmv_dtype { FLEXSPMV_F32 = 0, FLEXSPMV_F64 = 1, FLEXSPMV_I64 = 2 };
@@ -143,9 +149,10 @@ int flexspmv_last_kernel_ms(float* ms);
  *   out[2] snap_slack    ... unless 0 < t < num_tiles and the start of row (x & ~(snap_rows - 1)), x the
  *   out[3] snap_rows     row coordinate on that diagonal, is at most snap_slack merge items back: then the
  *                        boundary is that row start.  snap_slack = 0: boundaries stay on their diagonals.
- *   out[4] tile_capacity merge items a block can hold (nominal + snap_slack)
- *   out[5] search_in_blocks  1 when the reducer blocks search their own boundaries (no table is written
- *                        unless FLEXSPMV_FLAG_KEEP_TILES is given), else 0
+ *   out[4] tile_capacity merge items a block can hold (threads x items per thread of the policy); at least
+ *                        nominal + snap_slack, and more where a cap on the rows per tile shortens nominal
+ *   out[5] search_in_blocks  1 when the reducer blocks search their own boundaries instead of a search
+ *                        kernel (the tile table is left in the workspace either way), else 0
  * For libraries without a reducer the tiles are plain edge ranges of `nominal` edges.
  * Returns FLEXSPMV_OK, FLEXSPMV_ERR_BAD_DTYPE or FLEXSPMV_ERR_TOO_LARGE. */
 int flexspmv_tiling(int32_t dtype, int64_t num_rows, int64_t ne, int32_t out[6]);

@@ -18,7 +18,8 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, ROOT)
 
 BUILD_DIR = os.path.join(HERE, "_build")
-GRAPHS = ["csr_spmv", "spmv_dot", "spring_mass", "swe_rusanov", "system_two_selectors", "op_zoo"]
+GRAPHS = ["csr_spmv", "spmv_dot", "spring_mass", "swe_rusanov", "system_two_selectors", "op_zoo", "index_spmv",
+          "index_sums"]
 LARGE_ROUTE = ["-DFLEX_TUNE_INBLOCK_MAX_TILES=0", "-DFLEX_TUNE_SINGLE_FIXUP_MAX_TILES=0"]
 VARIANTS = {
     "large": {"policy": None, "flags": LARGE_ROUTE},

@@ -46,8 +46,9 @@ class OracleExtension:
                    and k != "row_end_offsets"}
         ro = bound["row_end_offsets"].numpy() if self.ir.has_reducer else None
         outs, after = run_oracle(self.ir, tensors, ro, bound["num_rows"], bound["num_cols"], num_threads=3)
-        for k, v in after.items():           # in-place map ops write through the inputs
-            bound[k].detach().view(-1)[:] = torch.from_numpy(v).view(-1)
+        for k, v in after.items():           # in-place map ops write through the inputs - through their memory, as
+            # a library does through raw pointers: torch sees no operation and bumps no version counter
+            np.copyto(bound[k].detach().numpy().reshape(-1), v.reshape(-1))
         return tuple(torch.from_numpy(o) for o in outs) if outs else None
 
 
@@ -612,3 +613,57 @@ def test_array_files_fail_loudly(tmp_path):
     save_mesh(mesh, bad)
     with pytest.raises(ValueError, match="outside"):
         load_mesh(bad)
+
+
+def test_edge_tensor_written_by_one_kernel_and_streamed_by_the_next_is_never_stale():
+    """Kernel A stores a per-edge tensor in place (through the raw pointer, not a torch operation); kernel B,
+    whose reducer ids are unsorted, streams that tensor through the edge permutation.  The wrapper keeps the
+    permuted copy of a streamed tensor only while the tensor is unchanged, so the store of A has to count as
+    a change: every call must see the fresh values."""
+    class TwoKernels(esr.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(5)
+            ne, nv, nr = 240, 30, 20
+            self.w = esr.Tensor(torch.rand(ne, generator=g, dtype=torch.float64))
+            self.v = esr.Tensor(torch.rand(nv, generator=g, dtype=torch.float64))
+            self.per_edge = esr.Tensor(torch.zeros(ne, dtype=torch.float64))
+            self.per_row = esr.Tensor(torch.zeros(nr, dtype=torch.float64))
+            self.per_row_2 = esr.Tensor(torch.zeros(nr, dtype=torch.float64))
+            self.pick = esr.Selector(torch.randint(0, nv, (ne,), generator=g))
+            rows = torch.randint(0, nr, (ne,), generator=g)                               # not sorted
+            ascending = torch.sort(rows).values
+            self.scatter = esr.Reducer(ascending, nr)                 # A: sorted ids, stores straight into per_edge
+            self.scatter_2 = esr.Reducer(rows, nr)                    # B: unsorted ids, streams through a permutation
+            self.row_of_edge = esr.Selector(ascending)
+
+        def forward(self):
+            prod = self.pick(self.v) * self.w
+            self.per_edge[:] = prod                                   # kernel A writes the edge tensor
+            self.per_row[:] = self.scatter(prod)
+            fresh = self.row_of_edge(self.per_row)                    # gather of A's result: kernel B starts here
+            self.per_row_2[:] = self.scatter_2(self.per_edge * fresh)  # B streams the tensor A wrote
+
+    eager, traced = TwoKernels(), TwoKernels()
+    [compiled] = esr.compile([traced], "torch")
+    exts, skipped = replace_all_with_oracle(compiled, "t_two_kernels")
+    assert not skipped and len(exts) >= 2
+    wrappers = [m for m in compiled.modules() if type(m).__name__ == "_DynamicCudaWrapper"]
+    assert any("per_edge" in w._written_inputs and w.edge_permutation is None for w in wrappers)
+    assert any("per_edge" in w._non_gather_value_inputs and "per_edge" not in w._written_inputs
+               and w.edge_permutation is not None for w in wrappers)
+    for step in range(3):
+        eager()
+        compiled()
+        assert torch.allclose(eager.per_row_2, traced.per_row_2, rtol=1e-13, atol=0), step
+        with torch.no_grad():                                         # other vertex data for the next step
+            eager.v.mul_(1.25)
+            traced.v.mul_(1.25)
+
+
+def test_permutation_into_a_given_tensor_counts_as_a_write():
+    from flexspmv_amd.formats import mark_written
+    t = torch.zeros(4)
+    before = t._version
+    mark_written(t)
+    assert t._version == before + 1

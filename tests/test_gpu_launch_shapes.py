@@ -40,7 +40,7 @@ def variant_extension(variant, name):
         if not os.path.exists(path):
             raise RuntimeError(f"{path} is not built: run __graft_entry__.build() "
                                "(or tests/launch_shapes/build_launch_shapes.py)")
-        _extensions[key] = HipExtension(path)
+        _extensions[key] = HipExtension(path, allow_variant=True)
     return _extensions[key]
 
 
@@ -79,6 +79,28 @@ def test_reducer_graphs_on_every_row_structure(variant, name, structure, dtype):
     tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get(name), dtype, rng, row_ptr=row_ptr)
     print(f"case {variant} {name} {structure} {np.dtype(dtype).name} rows={nr} ne={ne}", flush=True)
     parity.check_against_oracle(name, tensors, row_ptr, nr, nc, dtype)
+
+
+@pytest.mark.parametrize("structure", STRUCTURES)
+@pytest.mark.parametrize("name", parity.INT64_REDUCER_GRAPHS)
+def test_int64_reducers_and_aggregators_are_bit_exact(variant, name, structure):
+    """8-byte integers through the search kernel, fix-up blocks of 256 tiles (with runs that cross them on the
+    256-item tiles) and the final sum: bit for bit the oracle's."""
+    rng = parity.case_rng("launch shapes int64", name, structure)
+    row_ptr = row_structure(structure, rng)
+    tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get(name), np.int64, rng, row_ptr=row_ptr)
+    print(f"case {variant} {name} {structure} int64 rows={nr} ne={ne}", flush=True)
+    parity.check_against_oracle(name, tensors, row_ptr, nr, nc, np.int64)
+
+
+def test_int64_rows_that_carry_through_several_fixup_blocks(variant):
+    tile = 256 if variant == "tiny" else 2048
+    for name in parity.INT64_REDUCER_GRAPHS:
+        rng = parity.case_rng("long runs int64", name)
+        row_ptr = long_run_structure(rng, tile)
+        tensors, row_ptr, nr, nc, ne = make_inputs(graphs.get(name), np.int64, rng, row_ptr=row_ptr)
+        print(f"case {variant} long runs {name} int64 rows={nr} ne={ne}", flush=True)
+        parity.check_against_oracle(name, tensors, row_ptr, nr, nc, np.int64)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])

@@ -160,7 +160,7 @@ def test_launch_rejects_bad_arguments_without_touching_the_gpu():
     err = lambda: lib.flexspmv_last_error().decode()
     assert lib.flexspmv_launch(None) == -1
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, struct_size=8))) == -1 and "struct_size" in err()
-    assert lib.flexspmv_launch(ctypes.byref(_args(lib, flags=8))) == -1 and "flags" in err()
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, flags=16))) == -1 and "flags" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, num_value_inputs=1))) == -1 and "counts" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, dtype=2))) == -2 and "Unsupported dtype" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, ne=0))) == -1 and "non-empty" in err()
@@ -251,7 +251,102 @@ def test_launcher_keeps_its_previous_arguments_by_weak_reference_only():
     assert ext._same_arguments(tuple([args[0].clone()] + args[1:])) is None  # another tensor object
     args[1].resize_(2)
     assert ext._same_arguments(tuple(args)) is None                          # the same object in another state
+    args[1].resize_(4)
+    assert ext._same_arguments(tuple(args)) is not None
+    args[1].data = args[1].data.view(torch.int32)                            # same storage, size and layout: another dtype
+    assert ext._same_arguments(tuple(args)) is None
+    args[1].data = args[1].data.view(torch.float32)
+    assert ext._same_arguments(tuple(args)) is not None
     probe = weakref.ref(args[0])
     del args
     gc.collect()
     assert probe() is None
+
+
+def test_scratch_of_idle_streams_is_dropped():
+    """A caller that cycles through streams does not grow the launcher's scratch table without bound: beyond a
+    few entries, buffers of streams that have not launched for a while go - never one a capture recorded -
+    and a tile table remembered in a dropped buffer is forgotten with it."""
+    from flexspmv_amd.binding import HipExtension
+
+    class Probe(HipExtension):          # the bookkeeping alone, without a library or a GPU
+        def __init__(self):
+            self._workspace, self._last_used, self._captured, self._retained = {}, {}, set(), []
+            self._launch_count = 0
+            self._tile_key = None
+
+    class Buf:
+        def __init__(self, ptr):
+            self.ptr = ptr
+        def data_ptr(self):
+            return self.ptr
+        def numel(self):
+            return 256
+
+    ext = Probe()
+    for i in range(ext.MAX_IDLE_SCRATCH):
+        ext._workspace[(0, i)] = Buf(1000 + i)
+        ext._last_used[(0, i)] = 0
+    ext._captured.add((0, 3))
+    ext._tile_key = (1, 0, 10, 10, "float32", 1002, 0)      # table remembered in the buffer of stream 2
+    ext._launch_count = ext.IDLE_LAUNCHES - 1
+    ext._last_used[(0, 5)] = ext._launch_count                # stream 5 launched just now
+    ext._workspace[(0, 99)] = Buf(2000)
+    ext._drop_idle_scratch(keep=(0, 99))
+    assert len(ext._workspace) == ext.MAX_IDLE_SCRATCH + 1    # nothing is idle long enough yet
+    ext._launch_count += 1
+    ext._drop_idle_scratch(keep=(0, 99))
+    assert sorted(ext._workspace) == [(0, 3), (0, 5), (0, 99)]
+    assert ext._tile_key is None
+
+
+# ---------------------------------------------------------------------------------------------
+# tuning switches: a library built with them is a measurement variant and says so
+# ---------------------------------------------------------------------------------------------
+def test_every_tuning_switch_of_the_sources_is_listed_in_the_fence():
+    with open(os.path.join(build.CSRC_DIR, "flex_tuning.hpp")) as f:
+        listed = set(re.findall(r"defined\((FLEX_TUNE_[A-Z0-9_]+)\)", f.read()))
+    used = set()
+    for fn in os.listdir(build.CSRC_DIR):
+        if fn != "flex_tuning.hpp":
+            with open(os.path.join(build.CSRC_DIR, fn)) as f:
+                used |= set(re.findall(r"\bFLEX_TUNE_[A-Z0-9_]+", f.read()))
+    assert used and used <= listed, sorted(used - listed)
+
+
+def test_tuning_switches_are_recorded_and_variants_are_refused(tmp_path):
+    from flexspmv_amd.binding import HipExtension, variant_of
+    ir = graphs.get("csr_spmv")
+    _, sig = generate_hip_source(ir)
+    assert sig["tuning"] == [] and sig["policy_override"] == {} and variant_of(sig) == ""
+    src, sig = generate_hip_source(ir, policy={"block": 128, "ipt_f32": 4}, defines=["FLEX_TUNE_NT_LOADS", "FLEX_TUNE_NOMINAL=1024"])
+    assert sig["tuning"] == ["FLEX_TUNE_NOMINAL=1024", "FLEX_TUNE_NT_LOADS"]
+    assert variant_of(sig) == "FLEX_TUNE_NOMINAL=1024 FLEX_TUNE_NT_LOADS block=128 ipt_f32=4"
+    assert "#define FLEX_TUNING_DECLARED 1" in src
+    with pytest.raises(ValueError, match="not a tuning switch"):
+        generate_hip_source(ir, defines=["NDEBUG"])
+    # built through the package: switches reach the generator and the compiler alike, the signature names them,
+    # and only a caller that asks for a variant gets one
+    lib = build.compile_graph(ir, out_dir=str(tmp_path / "variant"), extra_flags=["-DFLEX_TUNE_NT_LOADS"])
+    assert json.loads(load_library(lib).flexspmv_signature().decode())["tuning"] == ["FLEX_TUNE_NT_LOADS"]
+    with pytest.raises(RuntimeError, match="measurement variant"):
+        HipExtension(lib)
+    assert HipExtension(lib, allow_variant=True).variant == "FLEX_TUNE_NT_LOADS"
+    for name in graphs.REGISTRY:                      # every shipped library is a product library
+        assert variant_of(json.loads(_lib(name).flexspmv_signature().decode())) == ""
+
+
+@pytest.mark.parametrize("flags, message", [
+    (["-DFLEX_TUNE_NT_LOADS"], "must be the ones the generator was given"),              # not declared to the generator
+    (["-DFLEX_TUNE_FORCE_MERGE"], "FLEX_TUNE_ALLOW_WRONG_RESULTS"),                      # wrong results need a second switch
+    (["-DFLEX_TUNE_ABLATE_STORES"], "FLEX_TUNE_ALLOW_WRONG_RESULTS"),
+    (["-DFLEX_TUNE_UNSAFE_BIG_TILE"], "FLEX_TUNE_ALLOW_WRONG_RESULTS"),
+])
+def test_undeclared_or_unsafe_switches_do_not_compile(tmp_path, flags, message):
+    import subprocess
+    ir = graphs.get("csr_spmv")
+    src, _ = build.write_generated_source(ir, out_dir=str(tmp_path))        # generated without switches
+    cmd = [build.hipcc_path(), *build.HIPCC_FLAGS, *flags, f"-I{build.CSRC_DIR}", f"-I{build.INCLUDE_DIR}",
+           "--cuda-host-only", "-fsyntax-only", src]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode != 0 and message in proc.stdout, proc.stdout[-2000:]

@@ -332,3 +332,71 @@ def test_op_zoo_oracle_equals_numpy_statement(dtype, tol):
         assert np.abs(o - ref[name]).max() <= tol * scale, name
     for name in ("acc", "dst6"):                       # in-place results written through the inputs
         assert np.abs(after[name] - ref[name]).max() <= tol * np.abs(ref[name]).max(), name
+
+
+# ---------------------------------------------------------------------------------------------
+# int64 sub-graphs with reducers and aggregators: integer sums have one right answer
+# ---------------------------------------------------------------------------------------------
+def _segment_sums(a, row_ptr):
+    """Exact per-row sums of an integer array [ne][Dim] (plain numpy, one row at a time)."""
+    a = a.reshape(len(a), -1)
+    out = np.zeros((len(row_ptr) - 1, a.shape[1]), dtype=np.int64)
+    for r in range(len(row_ptr) - 1):
+        out[r] = a[row_ptr[r]:row_ptr[r + 1]].sum(axis=0)
+    return out
+
+
+@pytest.mark.parametrize("T", [1, 3, 8, 64, 256])
+@pytest.mark.parametrize("structure", ["mesh_with_gaps", "skewed", "one_long_row", "mostly_empty", "tiny"])
+def test_int64_reducer_graphs_equal_exact_integer_sums(structure, T):
+    from tests.util_inputs import make_inputs, row_structure
+    rng = np.random.default_rng(33)
+    row_ptr = row_structure(structure, rng)
+    t, row_ptr, nr, nc, ne = make_inputs(graphs.get("index_spmv"), np.int64, rng, row_ptr=row_ptr)
+    (y, total), _ = run_oracle(graphs.get("index_spmv"), t, row_ptr, nr, nc, T)
+    prod = t["w"] * t["ids"][t["selector_idx"]]
+    assert y.dtype == np.int64 and np.array_equal(y, _segment_sums(prod, row_ptr)[:, 0])
+    assert np.array_equal(total, [prod.sum()])
+    t, row_ptr, nr, nc, ne = make_inputs(graphs.get("index_sums"), np.int64, rng, row_ptr=row_ptr)
+    (red, weight, total), _ = run_oracle(graphs.get("index_sums"), t, row_ptr, nr, nc, T)
+    mul = t["ids"][t["sel_idx"]] * t["w"][:, None]
+    rows = np.repeat(np.arange(nr), np.diff(row_ptr))
+    assert np.array_equal(red, _segment_sums(mul - t["ids"][rows], row_ptr))
+    assert np.array_equal(weight, _segment_sums(t["w"], row_ptr)[:, 0])
+    assert np.array_equal(total, mul.sum(axis=0))
+
+
+# ---------------------------------------------------------------------------------------------
+# the parity criterion itself: rounding differences pass, a wrong row does not
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name, dtype", [("spring_mass", np.float32), ("swe_rusanov", np.float64),
+                                         ("csr_spmv", np.float32), ("spmv_dot", np.float64)])
+def test_row_criterion_accepts_reordering_and_rejects_a_wrong_edge(name, dtype):
+    from oracle.parity import TOL, reducer_row_scales, row_excess
+    from tests.util_inputs import make_inputs, row_structure
+    rng = np.random.default_rng(44)
+    row_ptr = row_structure("mesh_with_gaps", rng)
+    ir = graphs.get(name)
+    t, row_ptr, nr, nc, ne = make_inputs(ir, dtype, rng, row_ptr=row_ptr)
+    tol = TOL[np.dtype(dtype)]
+    scales = reducer_row_scales(ir, t, row_ptr, nc, 4)
+    ref, _ = run_oracle(ir, t, row_ptr, nr, nc, 8)
+    other, _ = run_oracle(ir, t, row_ptr, nr, nc, 1)         # another summation order
+    # one edge of one row takes the value of its neighbour: a single wrong operand
+    streamed = next(k for k, v in t.items() if not k.endswith("_idx") and len(v) == ne)
+    bad_inputs = dict(t)
+    e = int(row_ptr[nr // 2])                                 # first edge of a row in the middle
+    assert row_ptr[nr // 2 + 1] > e
+    changed = t[streamed].copy()
+    changed[e] = changed[e] * 1.001
+    bad_inputs[streamed] = changed
+    wrong, _ = run_oracle(ir, bad_inputs, row_ptr, nr, nc, 8)
+    for i, (scale, floor) in scales.items():
+        assert row_excess(other[i], ref[i], tol, scale, floor).max() <= 1.0
+        assert row_excess(wrong[i], ref[i], tol, scale, floor).max() > 1.0
+        # the floor is a few ulps of the row's own terms, not a launch-wide constant
+        eps = np.finfo(dtype).eps
+        rows_with_edges = np.diff(row_ptr) > 0
+        assert np.all(floor[~rows_with_edges] == 0)
+        assert np.all(floor[rows_with_edges] <= 2000 * eps * np.maximum(scale[rows_with_edges], 1e-300) + 1e-300) \
+            or name in ("spring_mass", "swe_rusanov")         # maps with a cancellation inside are allowed more

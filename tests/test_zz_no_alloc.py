@@ -92,6 +92,47 @@ def test_static_scratch_launch_matches_the_allocating_one_twice_in_a_row(name, d
             assert torch.equal(o, w), f"{name}: static-scratch launch differs from flexspmv_launch (call {round_})"
 
 
+def test_static_scratch_launch_under_stream_capture():
+    """An allocation (or a free, or an event creation) under stream capture is an error, so a captured call
+    that succeeds and replays to the bits of flexspmv_launch made none.  The graph is replayed several
+    times with the program's own eager launches and synchronizations between the replays, and every replay
+    is checked (the scratch keeps what the eager launches in between left there)."""
+    name, dtype = "spmv_dot", "float64"
+    ext = load_named(name, build_if_missing=False)
+    rng = case_rng("no_alloc", "capture")
+    given, nr, nc, ne = device_inputs(ext, name, np.dtype(dtype), "skewed", rng)
+    other, onr, onc, one = device_inputs(ext, name, np.dtype(dtype), "mesh_with_gaps", rng)
+    want = ext.merged_spmv_launch(*[given[k] for k in ext.param_names()])
+    other_want = ext.merged_spmv_launch(*[other[k] for k in ext.param_names()])
+    outs = [torch.full_like(o, float("nan")) for o in want]
+    other_outs = [torch.full_like(o, float("nan")) for o in other_want]
+    rc, msg = launch_static(ext, given, nr, nc, ne, dtype, outs)       # resolves the scratch address outside the capture
+    assert rc == 0, msg
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            rc, msg = launch_static(ext, given, nr, nc, ne, dtype, outs)
+    assert rc == 0, msg
+    torch.cuda.current_stream().wait_stream(stream)
+    for replay in range(4):
+        for o in outs:
+            o.fill_(float("nan"))
+        # eager work of another shape through the same scratch between the replays
+        rc, msg = launch_static(ext, other, onr, onc, one, dtype, other_outs)
+        assert rc == 0, msg
+        torch.cuda.synchronize()
+        print(f"case no_alloc capture replay {replay}", flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, w in zip(outs, want):
+            assert torch.equal(o, w), f"replay {replay} differs from flexspmv_launch"
+        for o, w in zip(other_outs, other_want):
+            assert torch.equal(o, w)
+
+
 def test_static_scratch_launch_refuses_what_it_cannot_hold():
     ext = load_named("spmv_dot", build_if_missing=False)
     rng = case_rng("no_alloc", "limits")
