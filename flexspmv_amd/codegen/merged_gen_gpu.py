@@ -166,6 +166,11 @@ def _emit_map(op: Dict[str, Any], vars: Dict[str, Var], edge: str) -> List[str]:
         if float(e).is_integer() and 1 <= int(e) <= 4:
             return [f"{T} {name}(flex::v_ipow<{int(e)}>({a[0]}));" if scalar
                     else f"{T} {name} = {a[0]}.template ipow<{int(e)}>();"]
+    if o == "truediv" and isinstance(arg_name(op["args"][0]), str) and isinstance(arg_name(op["args"][1]), str):
+        num, den = vars.get(a[0]), vars.get(a[1])
+        if num is not None and den is not None and num.kind == "tensor" and num.dim > 1 and den.kind == "scalar":
+            # a tensor of several values over a scalar (a vector over its norm): one reciprocal, then products
+            return [f"{T} {name} = flex::times_reciprocal({a[0]}, {a[1]});"]
     if o in binary:
         return [f"{T} {name} = {a[0]} {binary[o]} {a[1]};"]
     if o == "neg":

@@ -386,8 +386,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   constexpr int RED = G::RED_WIDTH, AGG = G::AGG_WIDTH, ROW = G::ROW_WIDTH;
   constexpr int REDN = RED > 0 ? RED : 1;
   constexpr int FVN = FV > 0 ? FV : 1, FIN = FI > 0 ? FI : 1;
-  constexpr int OUT_CAP = TILE;               // merge path: every row a tile can finish is buffered in LDS
-  constexpr int OUT_STRIDE = OUT_CAP + WAVE;  // + one dump slot per lane for items that close no row
+  constexpr bool MAP_FIRST = (ROW == 0);  // merge path: the map runs before the walk (see below)
 #ifndef FLEX_TUNE_ROW_PATH_MAX_LEN
 #define FLEX_TUNE_ROW_PATH_MAX_LEN 32
 #endif
@@ -407,18 +406,28 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   static_assert(NWORDS <= WAVE, "one wavefront scans the bitmap words");
 #endif
 
-  // s_fv / s_fi hold what was fetched for the tile's edges, s_out the rows the merge path finishes.
-  // Where both fit a modest budget they are separate; otherwise s_out reuses s_fv after a barrier.
+  // LDS.  s_fv / s_fi hold what was fetched for the tile's edges, s_out one finished total per row end for the
+  // merge path (TILE rows: a tile may consist of row ends only), s_dump one slot per lane for items that
+  // close no row.  Where everything fits a modest budget s_out is a region of its own; otherwise it lies over
+  // s_fv and s_fi together - the walk has read its items from both by then - so that a block needs no more
+  // than the larger of the two.  The spring-mass map (two streamed values and an index per edge, three
+  // reduced values per row): 24.6 KB + the dump slots instead of 33.9 KB, 6 resident blocks per CU instead of 4.
 #ifndef FLEX_TUNE_SEPARATE_OUT_BYTES
 #define FLEX_TUNE_SEPARATE_OUT_BYTES (20 * 1024)
 #endif
-  constexpr int FV_ELEMS = FVN * TILE, OUT_ELEMS = REDN * OUT_STRIDE;
-  constexpr bool SEPARATE_OUT =
-      (size_t)(FV_ELEMS + OUT_ELEMS) * sizeof(V) + (size_t)FIN * TILE * 4 <= (size_t)FLEX_TUNE_SEPARATE_OUT_BYTES;
-  constexpr int LDS_ELEMS = SEPARATE_OUT ? FV_ELEMS + OUT_ELEMS : (FV_ELEMS > OUT_ELEMS ? FV_ELEMS : OUT_ELEMS);
-  __shared__ __attribute__((aligned(16))) V s_fv[LDS_ELEMS];
-  __shared__ __attribute__((aligned(16))) int s_fi[FIN * TILE];
-  V* const s_out = SEPARATE_OUT ? s_fv + FV_ELEMS : s_fv;
+  constexpr int FV_ELEMS = (MAP_FIRST && REDN * TILE > FVN * TILE) ? REDN * TILE : FVN * TILE;  // fetched data / contributions
+  constexpr size_t FV_BYTES = (size_t)FV_ELEMS * sizeof(V), FI_BYTES = (size_t)FIN * TILE * 4;
+  constexpr size_t OUT_BYTES = (size_t)REDN * TILE * sizeof(V), DUMP_BYTES = (size_t)REDN * WAVE * sizeof(V);
+  constexpr bool SEPARATE_OUT = FV_BYTES + FI_BYTES + OUT_BYTES + DUMP_BYTES <= (size_t)FLEX_TUNE_SEPARATE_OUT_BYTES;
+  constexpr size_t FETCH_BYTES = FV_BYTES + FI_BYTES;
+  constexpr size_t MAIN_BYTES = SEPARATE_OUT ? FETCH_BYTES + OUT_BYTES : (FETCH_BYTES > OUT_BYTES ? FETCH_BYTES : OUT_BYTES);
+  static_assert(FV_BYTES % 16 == 0 && FETCH_BYTES % 16 == 0 && MAIN_BYTES % 16 == 0, "LDS regions stay 16-byte aligned");
+  __shared__ __attribute__((aligned(16))) unsigned char s_raw[MAIN_BYTES + DUMP_BYTES];
+  V* const s_fv = reinterpret_cast<V*>(s_raw);
+  int* const s_fi = reinterpret_cast<int*>(s_raw + FV_BYTES);
+  V* const s_out = reinterpret_cast<V*>(s_raw + (SEPARATE_OUT ? FETCH_BYTES : 0));
+  // value c of row r at s_out[c * TILE + r]; value c of lane l's dump slot at s_out[DUMP_AT + c * WAVE + l]
+  constexpr int DUMP_AT = (int)((MAIN_BYTES - (SEPARATE_OUT ? FETCH_BYTES : 0)) / sizeof(V));
   __shared__ unsigned s_bits[NWORDS];
   __shared__ int s_vote[NW];
   __shared__ int s_wave_key[NW];
@@ -651,8 +660,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
     // gathers of a power-law matrix hit the same lines far more often than in per-thread item order) and
     // hand the contributions to the walk through LDS.  Graphs with row-aligned sources need the row of
     // every edge first: their walk takes the fetched data from LDS and gathers per item.
-    constexpr bool MAP_FIRST = (ROW == 0);
-    constexpr bool OUT_OVERLAPS = !SEPARATE_OUT || (MAP_FIRST && RED > FVN);  // s_out over data the walk reads
+    constexpr bool OUT_OVERLAPS = !SEPARATE_OUT;  // s_out lies over data the walk reads
     V* const s_x = s_fv;  // MAP_FIRST: contributions [c * TILE + j]; nobody reads s_fv after the vote
     if constexpr (MAP_FIRST) {
       const Pack<V, ROW> no_row{};
@@ -740,7 +748,6 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
 
     Pack<V, RED> tot;
     zero(tot);
-    const int dump = OUT_CAP + lane;
 #pragma unroll
     for (int it0 = 0; it0 < IPT; it0 += MERGE_CHUNK) {
       Gather ge[MERGE_CHUNK];
@@ -773,9 +780,8 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
         }
         // a row end parks the finished total in the output buffer (other items write a dump slot)
         {
-          const int slot = end ? xrel[it] : dump;
 #pragma unroll
-          for (int c = 0; c < RED; ++c) s_out[c * OUT_STRIDE + slot] = tot.v[c];
+          for (int c = 0; c < RED; ++c) s_out[end ? c * TILE + xrel[it] : DUMP_AT + c * WAVE + lane] = tot.v[c];
         }
 #pragma unroll
         for (int c = 0; c < RED; ++c) tot.v[c] = end ? V(0) : tot.v[c];
@@ -826,7 +832,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
     // (only this thread ever touches that row's slot, so a plain read-modify-write is safe)
     if (ends != 0u && in_key == xs) {
 #pragma unroll
-      for (int c = 0; c < RED; ++c) s_out[c * OUT_STRIDE + xs] += in_val[c];
+      for (int c = 0; c < RED; ++c) s_out[c * TILE + xs] += in_val[c];
     }
     // tile carry-out: what the tile accumulated for the row still open at its end
     if (tid == BLOCK - 1) {
@@ -848,7 +854,7 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
     for (int i = tid; i < R; i += BLOCK) {
       Pack<V, RED> t;
 #pragma unroll
-      for (int c = 0; c < RED; ++c) t.v[c] = s_out[c * OUT_STRIDE + i];
+      for (int c = 0; c < RED; ++c) t.v[c] = s_out[c * TILE + i];
       G::store_row(p, x0 + i, t);
     }
   }
