@@ -30,7 +30,7 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 from . import build as _build
 from .ir import FusedGraphIR
 
-ABI_VERSION = 5
+ABI_VERSION = 4
 FLAG_TIME_KERNEL = 1
 FLAG_REUSE_TILES = 2
 FLAG_KEEP_TILES = 4
@@ -38,7 +38,7 @@ FLAG_DEBUG_SYNC = 8
 DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
 EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
                     "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms", "flexspmv_tiling",
-                    "flexspmv_launch_static", "flexspmv_hot_capacity")
+                    "flexspmv_launch_static")
 
 
 class LaunchArgs(ctypes.Structure):
@@ -60,8 +60,6 @@ class LaunchArgs(ctypes.Structure):
         ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
         ("flags", ctypes.c_uint32),
-        ("hot_rows", ctypes.c_void_p),
-        ("num_hot_rows", ctypes.c_int32),
     ]
 
 
@@ -93,8 +91,6 @@ def load_library(path: str) -> ctypes.CDLL:
     lib.flexspmv_abi_version.restype = ctypes.c_int
     lib.flexspmv_tiling.argtypes = [ctypes.c_int32, ctypes.c_int64, ctypes.c_int64, ctypes.POINTER(ctypes.c_int32)]
     lib.flexspmv_tiling.restype = ctypes.c_int
-    lib.flexspmv_hot_capacity.argtypes = [ctypes.c_int32]
-    lib.flexspmv_hot_capacity.restype = ctypes.c_int
     if lib.flexspmv_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{path}: built for interface version {lib.flexspmv_abi_version()}, "
                            f"this package speaks {ABI_VERSION}")
@@ -176,10 +172,6 @@ class HipExtension:
         # Off by default: every launch then does all the work a launch of the reference does.
         self.reuse_tiles = False
         self._tile_key = None
-        # Rows of the gather source kept on chip by every launch (int32 tensor of row ids on the launch device, from
-        # flexspmv_amd.formats.encode_hot_rows, which also re-encodes the index tensor the launches must then
-        # be given), or None.  For power-law graphs; see include/flexspmv.h, flexspmv_launch_args.hot_rows.
-        self.hot_rows = None
         self.extra_flags = 0       # FLAG_* bits added to every launch (FLAG_DEBUG_SYNC: print every kernel's
                                    # grid / block / LDS on stderr and synchronize after it)
         # what a launch looks up, prepared once
@@ -205,10 +197,6 @@ class HipExtension:
         missing = [n for n in names if n not in bound]
         _check(not missing, f"merged_spmv_launch(): missing arguments {missing}")
         return bound
-
-    def hot_capacity(self, dtype: str) -> int:
-        """Most rows of the gather source a launch of this dtype can keep on chip (0: not supported)."""
-        return int(self._lib.flexspmv_hot_capacity(DTYPE_CODES[dtype]))
 
     def workspace_bytes(self, dtype: str, num_rows: int, ne: int) -> int:
         return int(self._lib.flexspmv_workspace_bytes(DTYPE_CODES[dtype], num_rows, ne))
@@ -451,19 +439,12 @@ class HipExtension:
         la.workspace, la.workspace_bytes = ws.data_ptr(), ws.numel()
         flags = (FLAG_TIME_KERNEL if self.time_kernel else 0) | int(self.extra_flags)
         if self.reuse_tiles and self._has_reducer:
-            key = (ro.data_ptr(), ro._version, num_rows, ne, dt, ws.data_ptr(), index, self.hot_rows is not None)
+            key = (ro.data_ptr(), ro._version, num_rows, ne, dt, ws.data_ptr(), index)
             if key == self._tile_key:
                 flags |= FLAG_REUSE_TILES
             self._tile_key = key
         la.flags = flags
         la.stream = raw_stream
-        hot = self.hot_rows
-        if hot is None:
-            la.hot_rows, la.num_hot_rows = None, 0
-        else:
-            if not (hot.is_cuda and hot.dtype == torch.int32 and hot.is_contiguous() and hot.device.index == index):
-                raise RuntimeError("hot_rows must be a contiguous int32 tensor on the launch device")
-            la.hot_rows, la.num_hot_rows = hot.data_ptr(), hot.numel()
         rc = self._lib.flexspmv_launch(st.ref)
         if rc != 0:
             raise RuntimeError(f"merged_spmv_launch failed ({rc}): {self._lib.flexspmv_last_error().decode()}")

@@ -303,27 +303,6 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
     value_streams = [f"if (q_w == {first}) return q_p.{target}_ptr;" for _, target, dim, first in kp.fetch_values
                      if fetch_contiguous]
     index_streams = [f"if (q_w == {slot}) return q_p.{module}_idx_ptr;" for module, slot in kp.fetch_indices]
-    # Launches that keep the most-gathered rows of the gather source in LDS (csrc/flex_wave_agent.hpp) need a
-    # graph that gathers one source through one selector and has no row-aligned sources.
-    hot_dim, hot_source = 0, "nullptr"
-    gather_cold_body, gather_table_body, pick_hot_body = [], [], []
-    if has_reducer and len(kp.gathers) == 1 and not kp.row_sources:
-        var, module, target, dim = kp.gathers[0]
-        T = kp.vars[var].ctype
-        hot_dim, hot_source = dim, f"q_p.{target}_ptr"
-        # entry ~i of a re-encoded index array (a negative number) names row i of the table of hot rows; its
-        # first q_lds rows are in LDS, the others are read from the (small, cache-resident) table in memory
-        gather_cold_body = [
-            f"const OffsetT q_i = q_f.index_{module};",
-            "const OffsetT q_t = (~q_i < q_lds) ? 0 : ~q_i;     // lanes served from LDS share one address",
-            f"const ValueT* q_src = (q_i >= 0) ? q_p.{target}_ptr + (size_t)q_i * {dim} : q_table + (size_t)q_t * {dim};",
-            f"q_g.{var} = {T}(q_src);"]
-        gather_table_body = [f"const OffsetT q_i = q_f.index_{module};",
-                             f"const HotTablePtr q_h = q_hot + ((q_i < 0 && ~q_i < q_lds) ? ~q_i : 0) * {dim};"] + \
-                            [f"q_g.{var}.values[{i}] = q_h[{i}];" for i in range(dim)]
-        pick_hot_body = [f"const bool q_in_lds = q_f.index_{module} < 0 && ~q_f.index_{module} < q_lds;"] + \
-                        [f"q_g.{var}.values[{i}] = q_in_lds ? q_table.{var}.values[{i}] : q_cold.{var}.values[{i}];"
-                         for i in range(dim)]
     load_row = []
     for var, target, dim, first in kp.row_sources:
         load_row += [f"q_rv.v[{first + i}] = q_p.{target}_ptr[(size_t)q_row * {dim} + {i}];" for i in range(dim)]
@@ -380,9 +359,6 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
         # what makes this library a measurement variant instead of a product library (both empty: product)
         "policy_override": {k: int(v) for k, v in sorted(policy.items())},
         "tuning": defines,
-        # index input whose entries may be re-encoded for launches with hot rows (None: not available)
-        "hot_index_input": (kp.gathers[0][1] + "_idx") if hot_dim else None,
-        "hot_source_input": kp.gathers[0][2] if hot_dim else None,
         "widths": {"fetch_values": kp.fetch_value_width, "fetch_indices": kp.fetch_index_width,
                    "reduce": kp.red_width, "aggregate": kp.agg_width, "row": kp.row_width},
     })
@@ -391,7 +367,7 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
 
     ctype = {"float32": "float", "float64": "double", "int64": "long"}
     enum = {"float32": "FLEXSPMV_F32", "float64": "FLEXSPMV_F64", "int64": "FLEXSPMV_I64"}
-    cases_run, cases_ws, cases_tiling, cases_static, cases_hot = [], [], [], [], []
+    cases_run, cases_ws, cases_tiling, cases_static = [], [], [], []
     for d in dtypes:
         disp = f"flex::Dispatch<Graph<{ctype[d]}>, {block}, {ipt[d]}, {'true' if has_reducer else 'false'}>"
         cases_run.append(
@@ -400,7 +376,6 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
             f"    case {enum[d]}: {{ Graph<{ctype[d]}>::Params p; Graph<{ctype[d]}>::fill(p, a); return {disp}::run_static(p, a); }}\n")
         cases_ws.append(f"    case {enum[d]}: return {disp}::workspace_bytes(num_rows, ne);\n")
         cases_tiling.append(f"    case {enum[d]}: return {disp}::tiling(num_rows, ne, out);\n")
-        cases_hot.append(f"    case {enum[d]}: return {disp}::hot_capacity();\n")
 
     src = f"""// Generated by flexspmv_amd.codegen.merged_gen_gpu for sub-graph "{ir.name}" ({ir.content_hash()}).
 // Do not edit: regenerate from the six-list description instead.
@@ -441,22 +416,6 @@ struct Graph {{
 {_indent(fetch_body)}  }}
   static FLEX_DEV void gather(const Params& q_p, const Fetch& q_f, Gather& q_g) {{
 {_indent(gather_body)}  }}
-  // gathers with the most-gathered rows of the source in an LDS table (0: not available for this sub-graph):
-  // an index entry < 0 names table row ~entry, any other entry the source row as usual
-  static constexpr int HOT_DIM = {hot_dim};
-  static FLEX_DEV const ValueT* hot_source(const Params& q_p) {{ return {hot_source}; }}
-  // Every lane does both loads - a lane whose row is in LDS reads row 0 of the table in memory (one address for
-  // all such lanes of a wavefront), the others LDS row 0 - and pick_hot selects afterwards: no load sits under a
-  // branch.  The
-  // table pointer is typed as an LDS pointer: with a generic one the compiler folds the two loads into one flat
-  // load from a selected address, which is slower than either and waits for everything in flight.
-  using HotTablePtr = const __attribute__((address_space(3))) ValueT*;
-  static FLEX_DEV void gather_cold(const Params& q_p, const Fetch& q_f, const ValueT* q_table, const int q_lds, Gather& q_g) {{
-{_indent(gather_cold_body)}  }}
-  static FLEX_DEV void gather_table(const Fetch& q_f, const HotTablePtr q_hot, const int q_lds, Gather& q_g) {{
-{_indent(gather_table_body)}  }}
-  static FLEX_DEV void pick_hot(const Fetch& q_f, const int q_lds, const Gather& q_cold, const Gather& q_table, Gather& q_g) {{
-{_indent(pick_hot_body)}  }}
   // the array behind streamed word q_w, where every streamed word is an array of its own
   static constexpr bool FETCH_CONTIGUOUS = {'true' if fetch_contiguous else 'false'};
   static FLEX_DEV const ValueT* value_stream(const Params& q_p, const int q_w) {{
@@ -514,12 +473,6 @@ int flexspmv_tiling(int32_t dtype, int64_t num_rows, int64_t ne, int32_t out[6])
   flex::g_last_error[0] = 0;
   switch (dtype) {{
 {''.join(cases_tiling)}    default: return flex::fail(FLEXSPMV_ERR_BAD_DTYPE, "Unsupported dtype for ValueT: this library was not generated for it");
-  }}
-}}
-
-int flexspmv_hot_capacity(int32_t dtype) {{
-  switch (dtype) {{
-{''.join(cases_hot)}    default: return 0;
   }}
 }}
 

@@ -16,7 +16,6 @@
 #include <mutex>
 
 #include "flex_agent.hpp"
-#include "flex_wave_agent.hpp"
 #include "flexspmv.h"
 
 // Scratch of flexspmv_launch_static: device memory that belongs to the library itself, so that entry point
@@ -244,145 +243,7 @@ struct Dispatch {
   static size_t workspace_bytes(int64_t num_rows, int64_t ne) {
     Layout l;
     if (!layout(num_rows, ne, l)) return 0;
-    HotLayout h;
-    if (HOT_CAPACITY > 0 && hot_layout(num_rows, ne, h) && h.total > l.total) return h.total;  // either kind of launch
     return l.total;
-  }
-
-  // ---- launches with hot rows: persistent wavefront tiles with the hot rows of the gather source in LDS ----
-  static constexpr int HOT_WAVES = 16, HOT_IPT = 8, HOT_MAX_GRID = 1024;
-  using HotTile = WaveTile<G, HOT_WAVES, HOT_IPT>;
-  static constexpr int HOT_CAPACITY = REDUCER ? HotTile::HOT_CAPACITY : 0;   // rows of the table that LDS holds
-  static constexpr int HOT_TABLE_ROWS = HOT_CAPACITY > 0 ? (1 << 20) : 1;    // rows of the table in all
-  struct HotLayout {
-    int num_tiles, carry_blocks;
-    size_t off_coords, off_carry_row, off_carry_val, off_table, off_partials, off_block_partials, total;
-  };
-  static bool hot_layout(int64_t num_rows, int64_t ne, HotLayout& h) {
-    const int64_t items = num_rows + ne;
-    if (items <= 0 || items >= ((int64_t)1 << 31) - TILE) return false;
-    constexpr int RED = G::RED_WIDTH > 0 ? G::RED_WIDTH : 1, AGG = G::AGG_WIDTH > 0 ? G::AGG_WIDTH : 1;
-    h.num_tiles = (int)((items + HotTile::WTILE - 1) / HotTile::WTILE);
-    h.carry_blocks = (h.num_tiles + FIXUP_BLOCK - 1) / FIXUP_BLOCK;
-    size_t off = 0;
-    h.off_coords = off;
-    off += align_up(sizeof(int2) * ((size_t)h.num_tiles + 1));
-    h.off_carry_row = off;
-    off += align_up(sizeof(int) * (size_t)h.num_tiles);
-    h.off_carry_val = off;
-    off += align_up(sizeof(V) * (size_t)h.num_tiles * RED);
-    h.off_table = off;
-    off += align_up(sizeof(V) * (size_t)HOT_TABLE_ROWS * HotTile::D);
-    h.off_partials = off;
-    off += align_up(sizeof(V) * (size_t)HOT_MAX_GRID * HOT_WAVES * AGG);
-    h.off_block_partials = off;
-    off += align_up(sizeof(V) * (size_t)h.carry_blocks * AGG);
-    h.total = off;
-    return true;
-  }
-  static int hot_capacity() { return HOT_CAPACITY; }
-
-  // one resident block per CU
-  static int hot_grid() {
-    static thread_local int cached_device = -1, cached = 0;
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess) return 8;
-    if (device != cached_device) {
-      int cus = 0;
-      if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0) cus = 256;
-      cached = cus < HOT_MAX_GRID ? cus : HOT_MAX_GRID;
-      cached_device = device;
-    }
-    return cached;
-  }
-
-  static int launch_hot(const typename G::Params& p, const flexspmv_launch_args* a, const HotLayout& h, char* ws) {
-    if constexpr (HOT_CAPACITY > 0) {
-      hipStream_t stream = (hipStream_t)a->stream;
-      const bool timed = (a->flags & FLEXSPMV_FLAG_TIME_KERNEL) != 0 && g_timer.ready();
-      if (timed) g_timer.armed = false;
-      const bool debug = (a->flags & FLEXSPMV_FLAG_DEBUG_SYNC) != 0 || debug_launch_env();
-      int debug_rc = FLEXSPMV_OK;
-      auto report = [&](const char* name, auto kernel, int grid, int block) {
-        if (debug && debug_rc == FLEXSPMV_OK) debug_rc = debug_report(name, kernel, (unsigned)grid, (unsigned)block, stream);
-      };
-      const int nnz = (int)a->ne, num_rows = (int)a->num_rows;
-      const int* row_end = a->row_end_offsets + 1;
-      int2* coords = (int2*)(ws + h.off_coords);
-      int* carry_row = (int*)(ws + h.off_carry_row);
-      V* carry_val = (V*)(ws + h.off_carry_val);
-      V* table = (V*)(ws + h.off_table);
-      V* partials = (V*)(ws + h.off_partials);
-      V* block_partials = (V*)(ws + h.off_block_partials);
-      if (debug)
-        fprintf(stderr, "[flexspmv] reducer launch with %d hot rows: %d rows, %d non-zeros, %d wavefront tiles of %d merge items, "
-                "%zu bytes of scratch\n", (int)a->num_hot_rows, num_rows, nnz, h.num_tiles, HotTile::WTILE, h.total);
-      Tiling tl;
-      tl.num_tiles = h.num_tiles;
-      tl.nominal = HotTile::WTILE;
-      tl.snap_slack = tl.snap_mask = tl.xcd_shift = tl.row_group = 0;
-      if ((a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0) {
-        constexpr int per_block = SEARCH_BLOCK / SEARCH_GROUP;
-        const int search_blocks = (h.num_tiles + 1 + per_block - 1) / per_block;
-        hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(SEARCH_BLOCK), 0, stream, tl, row_end, num_rows, nnz,
-                           coords);
-        report("tile_search_kernel", tile_search_kernel, search_blocks, SEARCH_BLOCK);
-      }
-      const int fill_blocks = ((int)a->num_hot_rows + 255) / 256;
-      hipLaunchKernelGGL((hot_fill_kernel<G>), dim3(fill_blocks), dim3(256), 0, stream, p, (const int*)a->hot_rows,
-                         (int)a->num_hot_rows, table);
-      report("hot_fill_kernel", hot_fill_kernel<G>, fill_blocks, 256);
-      const int grid = hot_grid();
-      auto kernel = wave_reduce_kernel<G, HOT_WAVES, HOT_IPT>;
-      if (timed) {
-        hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(HOT_WAVES * WAVE), 0, stream, g_timer.start, g_timer.stop, 0,
-                              (const int2*)coords, h.num_tiles, num_rows, row_end, nnz, p, carry_row, carry_val, partials,
-                              (const V*)table, (int)a->num_hot_rows);
-        g_timer.armed = true;
-      } else {
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(HOT_WAVES * WAVE), 0, stream, (const int2*)coords, h.num_tiles, num_rows,
-                           row_end, nnz, p, carry_row, carry_val, partials, (const V*)table, (int)a->num_hot_rows);
-      }
-      report("wave_reduce_kernel", kernel, grid, HOT_WAVES * WAVE);
-      // carries: the fix-up of the block tiles, which finds no aggregator partials per tile here ...
-      hipLaunchKernelGGL((fixup_kernel<G, FIXUP_BLOCK, 0, false>), dim3(h.carry_blocks), dim3(FIXUP_BLOCK), 0, stream, p,
-                         h.num_tiles, (const int*)carry_row, (const V*)carry_val, (const V*)partials, block_partials,
-                         (unsigned*)nullptr);
-      report("fixup_kernel", fixup_kernel<G, FIXUP_BLOCK, 0, false>, h.carry_blocks, FIXUP_BLOCK);
-      // ... aggregators: one partial per wavefront of the grid, added in wavefront order
-      if (G::AGG_WIDTH > 0) {
-        hipLaunchKernelGGL((aggregate_kernel<G, FIXUP_BLOCK>), dim3(1), dim3(FIXUP_BLOCK), 0, stream, p, (const V*)partials,
-                           grid * HOT_WAVES);
-        report("aggregate_kernel", aggregate_kernel<G, FIXUP_BLOCK>, 1, FIXUP_BLOCK);
-      }
-      const hipError_t e = hipGetLastError();
-      if (e != hipSuccess) return fail_hip(e, "kernel launch failed");
-      return debug_rc;
-    } else {
-      return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "this sub-graph does not support hot rows");
-    }
-  }
-
-  // hot rows given: the checks of that kind of launch; FLEXSPMV_OK with use_hot = false when none are given
-  static int check_hot(const flexspmv_launch_args* a, HotLayout& h, size_t workspace_bytes_available, bool& use_hot) {
-    use_hot = a->hot_rows != nullptr || a->num_hot_rows != 0;
-    if (!use_hot) return FLEXSPMV_OK;
-    if (HOT_CAPACITY <= 0)
-      return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "this sub-graph does not support hot rows (flexspmv_hot_capacity() is 0)");
-    if (a->hot_rows == nullptr || a->num_hot_rows <= 0 || a->num_hot_rows > HOT_TABLE_ROWS) {
-      snprintf(g_last_error, sizeof(g_last_error), "hot_rows needs between 1 and %d row ids, %d given", HOT_TABLE_ROWS,
-               (int)a->num_hot_rows);
-      return FLEXSPMV_ERR_BAD_ARGUMENT;
-    }
-    if (a->ne <= 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "selector index must be non-empty (ne > 0)");
-    if (a->num_rows <= 0) return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "num_rows must be positive");
-    if (!hot_layout(a->num_rows, a->ne, h))
-      return fail(FLEXSPMV_ERR_TOO_LARGE, "num_rows + ne must stay below 2^31 (32-bit offsets)");
-    if (h.total > workspace_bytes_available)
-      return fail(FLEXSPMV_ERR_WORKSPACE, "workspace is missing or smaller than flexspmv_workspace_bytes()");
-    if (a->row_end_offsets == nullptr)
-      return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "row_end_offsets is required by a reducer sub-graph");
-    return FLEXSPMV_OK;
   }
 
   static int tiling(int64_t num_rows, int64_t ne, int32_t* out) {
@@ -413,14 +274,8 @@ struct Dispatch {
   }
 
   static int run(const typename G::Params& p, const flexspmv_launch_args* a) {
-    const size_t available = a->workspace == nullptr ? 0 : a->workspace_bytes;
-    HotLayout h;
-    bool use_hot = false;
-    const int bad_hot = check_hot(a, h, available, use_hot);
-    if (bad_hot != FLEXSPMV_OK) return bad_hot;
-    if (use_hot) return launch_hot(p, a, h, (char*)a->workspace);
     Layout l;
-    const int bad = check(a, l, available);
+    const int bad = check(a, l, a->workspace == nullptr ? 0 : a->workspace_bytes);
     if (bad != FLEXSPMV_OK) return bad;
     return launch(p, a, l, (char*)a->workspace);
   }
@@ -429,13 +284,8 @@ struct Dispatch {
   static int run_static(const typename G::Params& p, const flexspmv_launch_args* a) {
     if ((a->flags & FLEXSPMV_FLAG_TIME_KERNEL) != 0)
       return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "FLEXSPMV_FLAG_TIME_KERNEL creates events; flexspmv_launch_static does not take it");
-    HotLayout h;
-    bool use_hot = false;
-    const int bad_hot = check_hot(a, h, l_unbounded(), use_hot);
-    if (bad_hot != FLEXSPMV_OK) return bad_hot;
     Layout l;
-    l.total = h.total;
-    const int bad = use_hot ? FLEXSPMV_OK : check(a, l, l_unbounded());
+    const int bad = check(a, l, l_unbounded());
     if (bad != FLEXSPMV_OK) return bad;
     if (l.total > (size_t)FLEXSPMV_STATIC_SCRATCH_BYTES) {
       snprintf(g_last_error, sizeof(g_last_error),
@@ -446,7 +296,6 @@ struct Dispatch {
     }
     char* ws = static_scratch();
     if (ws == nullptr) return FLEXSPMV_ERR_WORKSPACE;
-    if (use_hot) return launch_hot(p, a, h, ws);
     return launch(p, a, l, ws);
   }
   static constexpr size_t l_unbounded() { return ~(size_t)0; }

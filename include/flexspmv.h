@@ -20,7 +20,6 @@
  *   flexspmv_tiling           the tile arithmetic of the reference's dispatch (num_merge_tiles from
  *                             num_rows + num_nonzeros and the policy's tile size,
  *                             cuda_template/reducer/merged_spmv_template.cuh:60-80), as data.
- *   flexspmv_hot_capacity     no counterpart (see flexspmv_launch_args.hot_rows).
  *   flexspmv_last_kernel_ms   the GpuTimer bracket of the reference's CUDA harness
  *                             (src/flex_spmv_full_red.cu:298-330, utils.h:634-669), narrowed to the
  *                             dominant kernel of one launch so that a roofline can be measured live.
@@ -35,7 +34,7 @@
 extern "C" {
 #endif
 
-#define FLEXSPMV_ABI_VERSION 5
+#define FLEXSPMV_ABI_VERSION 4
 
 /* Scratch a library keeps for flexspmv_launch_static (bytes, per library and per GPU it is used on). */
 #define FLEXSPMV_STATIC_SCRATCH_BYTES (4u << 20)
@@ -91,13 +90,6 @@ enum flexspmv_status {
  *                  mean nothing to the caller; they only have to be left alone between two launches when
  *                  the second one carries FLEXSPMV_FLAG_REUSE_TILES.
  *   stream         hipStream_t to launch on (NULL = default stream).  The call is asynchronous.
- *   hot_rows       NULL, or num_hot_rows distinct row ids of the gather source (flexspmv_signature():
- *                  "hot_source_input") that the launch keeps in on-chip memory.  The index array named
- *                  "hot_index_input" must then be the re-encoded one (flexspmv_encode_hot_rows of
- *                  flexspmv_formats.h: entry ~i stands for hot_rows[i], other entries are unchanged).  Worth it
- *                  where a small share of the rows takes a large share of the gathers (power-law graphs);
- *                  num_hot_rows may not exceed flexspmv_hot_capacity().  Results are those of the launch
- *                  without hot rows up to the order of the sums.  No counterpart in the reference.
  */
 typedef struct flexspmv_launch_args {
   uint32_t struct_size; /* sizeof(flexspmv_launch_args) */
@@ -116,8 +108,6 @@ typedef struct flexspmv_launch_args {
   size_t workspace_bytes;
   void* stream;
   uint32_t flags; /* 0 or FLEXSPMV_FLAG_* */
-  const int32_t* hot_rows;
-  int32_t num_hot_rows;
 } flexspmv_launch_args;
 
 /* Run the fused sub-graph once.  Returns FLEXSPMV_OK, a negative flexspmv_status, or a hipError_t. */
@@ -166,11 +156,6 @@ int flexspmv_last_kernel_ms(float* ms);
  * For libraries without a reducer the tiles are plain edge ranges of `nominal` edges.
  * Returns FLEXSPMV_OK, FLEXSPMV_ERR_BAD_DTYPE or FLEXSPMV_ERR_TOO_LARGE. */
 int flexspmv_tiling(int32_t dtype, int64_t num_rows, int64_t ne, int32_t out[6]);
-
-/* Most rows a launch of this dtype can keep on chip (flexspmv_launch_args.hot_rows); 0 when the sub-graph does
- * not support hot rows (it must gather one source through one selector and have no row-aligned sources) or
- * the dtype is not compiled in.  No counterpart in the reference. */
-int flexspmv_hot_capacity(int32_t dtype);
 
 /* FLEXSPMV_ABI_VERSION the library was built against. */
 int flexspmv_abi_version(void);
