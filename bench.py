@@ -364,7 +364,14 @@ def time_edge_list_preparation(w, steps):
                               b / ms / 1e6 / HBM_PEAK_GBS, "matches_generator": ok}
     shuffled = rows[torch.randperm(ne, device="cuda")]
     ms = timed(lambda: formats.sort_edges_by_row(shuffled, nr), max(1, steps // 10))
-    out["sort_edges_by_row"] = {"ms": ms, "edges_per_s": ne / ms * 1e3}
+    # radix sort, 8-bit digits over the bits of num_rows - 1; per digit the ids are read twice (counted, then moved
+    # with their positions) and written once: 4 + 8 + 8 bytes per edge, the first digit 4 + 4 + 8 (positions implicit)
+    digits = -(-max(1, (nr - 1).bit_length()) // 8)
+    b = ne * (16 + 20 * (digits - 1))
+    out["sort_edges_by_row"] = {"ms": ms, "edges_per_s": ne / ms * 1e3, "digits": digits, "algorithmic_bytes": b,
+                                "gbs": b / ms / 1e6, "frac_of_hbm_peak": b / ms / 1e6 / HBM_PEAK_GBS,
+                                "torch_stable_sort_ms": timed(lambda: torch.sort(shuffled, stable=True),
+                                                              max(1, steps // 10))}
     _, perm = formats.sort_edges_by_row(shuffled, nr)
     vals = torch.from_numpy(next(v for v in w.tensors.values() if v.dtype.kind == "f" and v.shape[0] == ne)).cuda()
     dst = torch.empty_like(vals)

@@ -295,7 +295,7 @@ def generate_hip_source(ir: FusedGraphIR, dtypes: Optional[Sequence[str]] = None
     for var, module, target, dim in kp.gathers:
         T = kp.vars[var].ctype
         gather_members.append(f"{T} {var};")
-        gather_body.append(f"q_g.{var} = {T}(q_p.{target}_ptr + (size_t)q_f.index_{module} * {dim});")
+        gather_body.append(f"q_g.{var} = {T}::gathered(q_p.{target}_ptr + (size_t)q_f.index_{module} * {dim});")
         body.append(f"{T} {var} = q_g.{var};")
     # every streamed word an array of its own (edge tensors of width 1, index arrays): a tile's slice of it
     # can then be copied as it lies in memory

@@ -14,13 +14,15 @@
 //   rows_search_kernel   the fallback for edge lists with huge runs of empty rows: one binary search per
 //                        row.  It is always launched and returns at once unless the first kernel asked for it,
 //                        so the host never has to look at device memory.
-//   sort                 rocPRIM's radix sort on (row id, position) pairs over the bits num_rows needs.
+//   sort_*_kernel        stable radix sort of (row id, position) pairs over the bits num_rows needs: per
+//                        8-bit digit a histogram per block, a scan, and a scatter that ranks with wave64
+//                        ballots and orders a tile in LDS so that every digit's run leaves as one piece.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
 
-#include <rocprim/rocprim.hpp>
+#include <type_traits>
 
 #include "flexspmv_formats.h"
 
@@ -140,8 +142,23 @@ rows_search_kernel(const I* __restrict__ rows, const int ne, const int num_rows,
   }
 }
 
-// key of a row id for the sort: ids that do not fit a non-negative int32 become 0xffffffff, which reads
-// back as -1 in sorted_rows and is reported as out of range by the pointer kernel
+// ---------------------------------------------------------------------------------------------------
+// Stable sort of (row id, position) pairs: least-significant-digit radix sort, 8-bit digits over the
+// bits num_rows needs.  Three kernels per digit, no atomics on memory and nothing to clear beforehand:
+//   sort_histogram_kernel   block b counts the digits of its chunk of tiles -> hist[digit][b]
+//   sort_scan_kernel        block d turns row d of hist into exclusive prefixes and leaves the row's sum
+//   sort_scatter_kernel     block b ranks its tiles' items (wave64 ballots give every item the lanes that
+//                           hold the same digit; wavefront counters in LDS carry the order across the 16
+//                           items of a lane and across the 4 wavefronts), orders a tile by digit in LDS
+//                           and writes each digit's run to its place: neighbouring lanes write
+//                           neighbouring words.
+// Position order inside a tile is wavefront-major: item k of lane l of wavefront w is element
+// w * 1024 + k * 64 + l, so every load is a whole 256-byte piece per wavefront.
+// Bytes per edge and digit: 4 read by the histogram, 8 read + 8 written by the scatter (the first digit
+// reads the caller's ids instead, 4 or 8 bytes, and no positions: they are the element numbers).
+
+// key of a row id: ids that do not fit a non-negative int32 become 0xffffffff, which reads back as -1 in
+// sorted_rows and is reported as out of range by the pointer kernel
 template <typename I>
 struct RowKey {
   __host__ __device__ unsigned operator()(const I v) const {
@@ -149,20 +166,359 @@ struct RowKey {
   }
 };
 
-int bits_for(int64_t num_rows) {
-  int b = 1;
-  while (b < 32 && ((int64_t)1 << b) < num_rows) ++b;
-  return b;
+constexpr int RADIX_BITS = 8;
+constexpr int RADIX = 1 << RADIX_BITS;
+constexpr int SORT_ITEMS = 16;                          // per thread and tile
+constexpr int SORT_WAVES = BLOCK / WAVE;
+constexpr int COUNT_TILE = BLOCK * SORT_ITEMS;          // the histogram's blocks: 256 threads, 4096 ids at a time
+// The scatter's blocks: 1024 threads and tiles of 16384 pairs for long lists (a digit's run of a tile is then
+// 64 pairs on average, two whole lines: 117 M pairs take 2.25 ms against 2.9 with tiles of 4096), 256 threads
+// and tiles of 4096 pairs where such tiles would leave the CUs a handful each (6 M pairs: 0.13 against 0.17 ms).
+constexpr int BIG_SCATTER_BLOCK = 1024;
+constexpr long long BIG_SCATTER_FROM = 16ll << 20;   // pairs
+constexpr int SORT_MAX_BLOCKS = 4096;                   // a block takes several tiles beyond that many
+constexpr int SORT_SCAN_ITEMS = SORT_MAX_BLOCKS / BLOCK;
+constexpr int SORT_MAX_PASSES = 4;
+static_assert(RADIX == BLOCK && BIG_SCATTER_BLOCK % BLOCK == 0, "thread d < 256 of a block owns digit d");
+
+// Ids outside [0, num_rows) sort as the last row, num_rows - 1 (a digit more for them would cost a whole
+// pass where num_rows is a power of two): they end up among that row's edges, in their original order,
+// and keep their value in sorted_rows, where the pointer kernel finds them.
+__device__ inline unsigned sort_digit(const unsigned key, const unsigned last_row, const int shift, const unsigned mask) {
+  return ((key < last_row ? key : last_row) >> shift) & mask;
+}
+
+template <typename I, bool FIRST>
+__device__ inline unsigned load_sort_key(const void* src, const long long i) {
+  if (FIRST) return RowKey<I>()(reinterpret_cast<const I*>(src)[i]);
+  return reinterpret_cast<const unsigned*>(src)[i];
+}
+
+__device__ inline unsigned wave_inclusive_sum(unsigned v, const int lane) {
+#pragma unroll
+  for (int off = 1; off < WAVE; off <<= 1) {
+    const unsigned other = __shfl_up(v, off);
+    if (lane >= off) v += other;
+  }
+  return v;
+}
+
+// Exclusive prefix of v over the block's WAVES wavefronts and the block's sum.  Two barriers; s_tmp holds
+// WAVES words and is free again on return.
+template <int WAVES>
+__device__ inline unsigned block_exclusive_sum(const unsigned v, unsigned* s_tmp, unsigned& total) {
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+  const unsigned inclusive = wave_inclusive_sum(v, lane);
+  if (lane == WAVE - 1) s_tmp[wave] = inclusive;
+  __syncthreads();
+  unsigned before = 0;
+  total = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    const unsigned s = s_tmp[w];
+    if (w < wave) before += s;
+    total += s;
+  }
+  __syncthreads();
+  return before + inclusive - v;
+}
+
+template <typename I, bool FIRST>
+__global__ void __launch_bounds__(BLOCK)
+sort_histogram_kernel(const void* __restrict__ keys_in, const long long ne, const unsigned last_row, const int shift,
+                      const unsigned mask, const int tiles_per_block, const int blocks, unsigned* __restrict__ hist) {
+  __shared__ unsigned s_cnt[SORT_WAVES][RADIX];
+  const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+#pragma unroll
+  for (int j = 0; j < RADIX / WAVE; ++j) s_cnt[wave][lane + j * WAVE] = 0;   // the wavefront's own counters
+  const long long first_tile = (long long)blockIdx.x * tiles_per_block;
+  for (int tl = 0; tl < tiles_per_block; ++tl) {
+    const long long base = (first_tile + tl) * COUNT_TILE + wave * (WAVE * SORT_ITEMS);
+    if (base >= ne) break;
+    unsigned key[SORT_ITEMS];
+#pragma unroll
+    for (int k = 0; k < SORT_ITEMS; ++k) {
+      const long long i = base + k * WAVE + lane;
+      key[k] = load_sort_key<I, FIRST>(keys_in, i < ne ? i : ne - 1);
+    }
+#pragma unroll
+    for (int k = 0; k < SORT_ITEMS; ++k) {
+      const bool valid = base + k * WAVE + lane < ne;
+      const unsigned d = sort_digit(key[k], last_row, shift, mask);
+      // a wavefront whose items all hold one digit (sorted input, a hot row, the high digit of small
+      // ids) adds once instead of 64 times to one counter
+      const unsigned d0 = __builtin_amdgcn_readfirstlane(d);
+      const unsigned long long active = __builtin_amdgcn_ballot_w64(valid);
+      const unsigned long long same = __builtin_amdgcn_ballot_w64(valid && d == d0);
+      if (same == active) {
+        if (lane == 0 && active != 0ull) atomicAdd(&s_cnt[wave][d0], (unsigned)__builtin_popcountll(active));
+      } else if (valid) {
+        atomicAdd(&s_cnt[wave][d], 1u);
+      }
+    }
+  }
+  __syncthreads();
+  unsigned sum = 0;
+#pragma unroll
+  for (int w = 0; w < SORT_WAVES; ++w) sum += s_cnt[w][threadIdx.x];
+  hist[(size_t)threadIdx.x * blocks + blockIdx.x] = sum;
+}
+
+__global__ void __launch_bounds__(BLOCK)
+sort_scan_kernel(unsigned* __restrict__ hist, const int blocks, unsigned* __restrict__ totals) {
+  __shared__ unsigned s_tmp[SORT_WAVES];
+  unsigned* row = hist + (size_t)blockIdx.x * blocks;
+  const int per = (blocks + BLOCK - 1) / BLOCK;   // <= SORT_SCAN_ITEMS
+  const int lo = threadIdx.x * per;
+  unsigned v[SORT_SCAN_ITEMS];
+  unsigned sum = 0;
+#pragma unroll
+  for (int j = 0; j < SORT_SCAN_ITEMS; ++j) {
+    v[j] = (j < per && lo + j < blocks) ? row[lo + j] : 0u;
+    sum += v[j];
+  }
+  unsigned total;
+  unsigned run = block_exclusive_sum<SORT_WAVES>(sum, s_tmp, total);
+#pragma unroll
+  for (int j = 0; j < SORT_SCAN_ITEMS; ++j) {
+    if (j < per && lo + j < blocks) row[lo + j] = run;
+    run += v[j];
+  }
+  if (threadIdx.x == 0) totals[blockIdx.x] = total;
+}
+
+// LDS of a scatter block of THREADS threads
+template <int THREADS>
+struct ScatterShared {
+  static constexpr int TILE = THREADS * SORT_ITEMS, WAVES = THREADS / WAVE;
+  unsigned keys[TILE];
+  int32_t vals[TILE];
+  unsigned cnt[WAVES][RADIX];
+  unsigned place[RADIX];   // where digit d's run of this tile goes, minus the run's start inside the tile
+  unsigned tmp[WAVES];
+};
+
+// One tile of `count` pairs starting at element tile_at.  FULL: count == THREADS * 16, no lane is idle.
+// next_of_digit (thread t < 256: digit t) is where the block's next item of that digit goes; advanced here.
+template <typename I, bool FIRST, bool FULL, int THREADS>
+__device__ inline void scatter_tile(ScatterShared<THREADS>& sh, const void* __restrict__ keys_in,
+                                    const int32_t* __restrict__ vals_in, unsigned* __restrict__ keys_out,
+                                    int32_t* __restrict__ vals_out, const long long tile_at, const int count,
+                                    const unsigned last_row, const int shift, const unsigned mask,
+                                    unsigned& next_of_digit) {
+  const int t = threadIdx.x, lane = t & (WAVE - 1), wave = t / WAVE;
+  const int first_pos = wave * (WAVE * SORT_ITEMS) + lane;   // item k of this lane is element first_pos + 64 k
+  unsigned key[SORT_ITEMS];
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; ++k) {
+    const int pos = first_pos + k * WAVE;
+    key[k] = load_sort_key<I, FIRST>(keys_in, tile_at + ((FULL || pos < count) ? pos : 0));
+  }
+#pragma unroll
+  for (int j = 0; j < RADIX / WAVE; ++j) sh.cnt[wave][lane + j * WAVE] = 0;
+  // Per item, among the wavefront's 64 items of step k: its digit (bits 0-7), how many of them hold the same
+  // digit (8-14), how many of those sit in lower lanes (16-21) and the lowest lane that holds it (24-29).
+  // Arithmetic only: per bit of the digit, keep the lanes whose bit equals this lane's.
+  unsigned info[SORT_ITEMS];
+  const unsigned below_lo = lane < 32 ? (1u << lane) - 1u : 0xffffffffu;
+  const unsigned below_hi = lane < 32 ? 0u : (1u << (lane - 32)) - 1u;
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; ++k) {
+    const bool valid = FULL || first_pos + k * WAVE < count;
+    const unsigned d = sort_digit(key[k], last_row, shift, mask);
+    const unsigned long long active = FULL ? ~0ull : __builtin_amdgcn_ballot_w64(valid);
+    unsigned peers_lo = (unsigned)active, peers_hi = (unsigned)(active >> 32);
+#pragma unroll
+    for (int b = 0; b < RADIX_BITS; ++b) {
+      const int all_if_set = (int)(d << (31 - b)) >> 31;   // -1 where bit b of the digit is set, else 0
+      const unsigned long long with_bit = __builtin_amdgcn_ballot_w64(all_if_set != 0);
+      peers_lo &= ~((unsigned)with_bit ^ (unsigned)all_if_set);
+      peers_hi &= ~((unsigned)(with_bit >> 32) ^ (unsigned)all_if_set);
+    }
+    const unsigned same = (unsigned)(__builtin_popcount(peers_lo) + __builtin_popcount(peers_hi));
+    const unsigned below = (unsigned)(__builtin_popcount(peers_lo & below_lo) + __builtin_popcount(peers_hi & below_hi));
+    const unsigned lowest = peers_lo != 0u ? (unsigned)__builtin_ctz(peers_lo) : 32u + (unsigned)__builtin_ctz(peers_hi);
+    info[k] = valid ? (d | (same << 8) | (below << 16) | (lowest << 24)) : (d | ((unsigned)lane << 24));
+    // finished here, one item at a time: left alone the compiler moves this arithmetic down to where info
+    // is used and keeps the 128 lane masks of the ballots until then
+    asm volatile("" : "+v"(info[k]));
+  }
+  // the positions travel with the keys; loaded here, they arrive while the counters are walked
+  int32_t val[SORT_ITEMS];
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; ++k) {
+    const int pos = first_pos + k * WAVE;
+    const long long i = tile_at + ((FULL || pos < count) ? pos : 0);
+    val[k] = FIRST ? (int32_t)i : vals_in[i];
+  }
+  // The lowest lane of every group moves the group's counter, step after step; every lane of the group
+  // reads the value from before: its rank among the wavefront's items of that digit, in position order.
+  unsigned digit_rank[SORT_ITEMS];
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; ++k) {
+    const unsigned d = info[k] & 0xffu, same = (info[k] >> 8) & 0xffu, below = (info[k] >> 16) & 0xffu;
+    const int lowest = (int)(info[k] >> 24);
+    unsigned old = 0;
+    if (lane == lowest && same != 0u) {
+      old = sh.cnt[wave][d];
+      sh.cnt[wave][d] = old + same;
+    }
+    old = __shfl(old, lowest);
+    digit_rank[k] = d | ((old + below) << RADIX_BITS);
+  }
+  __syncthreads();
+  {
+    // thread t < 256: digit t's items per wavefront -> start of every wavefront's share inside the tile
+    unsigned sum = 0;
+    if (t < RADIX) {
+#pragma unroll
+      for (int w = 0; w < THREADS / WAVE; ++w) sum += sh.cnt[w][t];
+    }
+    unsigned unused;
+    unsigned start = block_exclusive_sum<THREADS / WAVE>(sum, sh.tmp, unused);
+    if (t < RADIX) {
+      sh.place[t] = next_of_digit - start;   // modulo 2^32: the item at tile position i goes to place[d] + i
+      next_of_digit += sum;
+#pragma unroll
+      for (int w = 0; w < THREADS / WAVE; ++w) {
+        const unsigned c = sh.cnt[w][t];
+        sh.cnt[w][t] = start;
+        start += c;
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < SORT_ITEMS; ++k) {
+    if (FULL || first_pos + k * WAVE < count) {
+      const unsigned at = sh.cnt[wave][digit_rank[k] & (RADIX - 1)] + (digit_rank[k] >> RADIX_BITS);
+      sh.keys[at] = key[k];
+      sh.vals[at] = val[k];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int m = 0; m < SORT_ITEMS; ++m) {
+    const int i = t + m * THREADS;
+    if (FULL || i < count) {
+      const unsigned key_i = sh.keys[i];
+      const unsigned to = sh.place[sort_digit(key_i, last_row, shift, mask)] + (unsigned)i;
+      keys_out[to] = key_i;
+      vals_out[to] = sh.vals[i];
+    }
+  }
+  __syncthreads();
+}
+
+template <typename I, bool FIRST, int THREADS>
+__global__ void __launch_bounds__(THREADS)
+sort_scatter_kernel(const void* __restrict__ keys_in, const int32_t* __restrict__ vals_in,
+                    unsigned* __restrict__ keys_out, int32_t* __restrict__ vals_out, const long long ne,
+                    const unsigned last_row, const int shift, const unsigned mask, const int tiles_per_block,
+                    const int blocks, const unsigned* __restrict__ hist, const unsigned* __restrict__ totals) {
+  constexpr int TILE = THREADS * SORT_ITEMS;
+  __shared__ ScatterShared<THREADS> sh;
+  const int t = threadIdx.x;
+  // thread t follows digit t: the digit's place in the output, then this block's place among the blocks
+  unsigned unused;
+  unsigned next_of_digit = block_exclusive_sum<THREADS / WAVE>(t < RADIX ? totals[t] : 0u, sh.tmp, unused);
+  if (t < RADIX) next_of_digit += hist[(size_t)t * blocks + blockIdx.x];
+  const long long first_tile = (long long)blockIdx.x * tiles_per_block;
+  for (int tl = 0; tl < tiles_per_block; ++tl) {
+    const long long tile_at = (first_tile + tl) * TILE;
+    if (tile_at >= ne) break;   // the whole block leaves together
+    if (ne - tile_at >= TILE)
+      scatter_tile<I, FIRST, true, THREADS>(sh, keys_in, vals_in, keys_out, vals_out, tile_at, TILE, last_row, shift,
+                                            mask, next_of_digit);
+    else
+      scatter_tile<I, FIRST, false, THREADS>(sh, keys_in, vals_in, keys_out, vals_out, tile_at, (int)(ne - tile_at),
+                                             last_row, shift, mask, next_of_digit);
+  }
+}
+
+// What a sort of ne pairs with ids below num_rows runs: digits, chunks and the scratch layout.
+struct SortPlan {
+  int passes;
+  int shift[SORT_MAX_PASSES], bits[SORT_MAX_PASSES];
+  int scatter_threads;            // BIG_SCATTER_BLOCK or BLOCK
+  int tiles_per_block, blocks;    // scatter tiles (scatter_threads * 16 pairs) per block; blocks of both kernels
+  size_t off_keys, off_vals, off_hist, off_totals, bytes;
+};
+
+SortPlan plan_sort(int64_t ne, int64_t num_rows) {
+  SortPlan p{};
+  int key_bits = 1;   // enough for num_rows - 1
+  while (key_bits < 31 && ((int64_t)1 << key_bits) < num_rows) ++key_bits;
+  p.passes = (key_bits + RADIX_BITS - 1) / RADIX_BITS;
+  int shift = 0;
+  for (int i = 0; i < p.passes; ++i) {
+    p.bits[i] = key_bits / p.passes + (i < key_bits % p.passes ? 1 : 0);
+    p.shift[i] = shift;
+    shift += p.bits[i];
+  }
+  p.scatter_threads = ne >= BIG_SCATTER_FROM ? BIG_SCATTER_BLOCK : BLOCK;
+  const int64_t tile = (int64_t)p.scatter_threads * SORT_ITEMS;
+  const int64_t tiles = (ne + tile - 1) / tile;
+  p.tiles_per_block = (int)((tiles + SORT_MAX_BLOCKS - 1) / SORT_MAX_BLOCKS);
+  if (p.tiles_per_block < 1) p.tiles_per_block = 1;
+  p.blocks = (int)((tiles + p.tiles_per_block - 1) / p.tiles_per_block);
+  auto aligned = [](size_t n) { return (n + 255) & ~(size_t)255; };
+  size_t at = 0;
+  p.off_keys = at;   at += p.passes > 1 ? aligned((size_t)ne * 4) : 0;   // the second pair of buffers
+  p.off_vals = at;   at += p.passes > 1 ? aligned((size_t)ne * 4) : 0;
+  p.off_hist = at;   at += aligned((size_t)RADIX * p.blocks * 4);
+  p.off_totals = at; at += aligned((size_t)RADIX * 4);
+  p.bytes = at;
+  return p;
 }
 
 template <typename I>
-hipError_t sort_pairs(void* temp, size_t& temp_bytes, const I* rows, int32_t* sorted_rows, int32_t* permutation,
+hipError_t sort_pairs(const SortPlan& p, void* workspace, const I* rows, int32_t* sorted_rows, int32_t* permutation,
                       int64_t ne, int64_t num_rows, hipStream_t stream) {
-  auto keys_in = rocprim::make_transform_iterator(rows, RowKey<I>());
-  rocprim::counting_iterator<int32_t> positions(0);
-  // ids past num_rows keep their high bits out of the sort; they are reported, not ordered
-  return rocprim::radix_sort_pairs(temp, temp_bytes, keys_in, reinterpret_cast<unsigned*>(sorted_rows), positions,
-                                   permutation, (size_t)ne, 0u, (unsigned)bits_for(num_rows), stream);
+  char* ws = static_cast<char*>(workspace);
+  unsigned* alt_keys = reinterpret_cast<unsigned*>(ws + p.off_keys);
+  int32_t* alt_vals = reinterpret_cast<int32_t*>(ws + p.off_vals);
+  unsigned* hist = reinterpret_cast<unsigned*>(ws + p.off_hist);
+  unsigned* totals = reinterpret_cast<unsigned*>(ws + p.off_totals);
+  const void* keys_in = rows;
+  const int32_t* vals_in = nullptr;
+  for (int i = 0; i < p.passes; ++i) {
+    // the last digit writes the caller's arrays, the ones before it alternate so that it can
+    const bool to_caller = ((p.passes - 1 - i) & 1) == 0;
+    unsigned* keys_out = to_caller ? reinterpret_cast<unsigned*>(sorted_rows) : alt_keys;
+    int32_t* vals_out = to_caller ? permutation : alt_vals;
+    const unsigned mask = (1u << p.bits[i]) - 1u;
+    const dim3 grid((unsigned)p.blocks), block(BLOCK);
+    const unsigned last_row = (unsigned)(num_rows - 1);
+    // a block of the histogram counts the pairs the scatter's block of the same number moves
+    const int count_tiles = p.tiles_per_block * (p.scatter_threads * SORT_ITEMS / COUNT_TILE);
+    if (i == 0) {
+      hipLaunchKernelGGL((sort_histogram_kernel<I, true>), grid, block, 0, stream, keys_in, (long long)ne, last_row,
+                         p.shift[i], mask, count_tiles, p.blocks, hist);
+    } else {
+      hipLaunchKernelGGL((sort_histogram_kernel<int32_t, false>), grid, block, 0, stream, keys_in, (long long)ne,
+                         last_row, p.shift[i], mask, count_tiles, p.blocks, hist);
+    }
+    hipLaunchKernelGGL(sort_scan_kernel, dim3(RADIX), block, 0, stream, hist, p.blocks, totals);
+    auto scatter = [&](auto first, auto threads) {
+      constexpr bool FIRST = decltype(first)::value;
+      constexpr int THREADS = decltype(threads)::value;
+      using Id = typename std::conditional<FIRST, I, int32_t>::type;
+      hipLaunchKernelGGL((sort_scatter_kernel<Id, FIRST, THREADS>), grid, dim3(THREADS), 0, stream, keys_in, vals_in,
+                         keys_out, vals_out, (long long)ne, last_row, p.shift[i], mask, p.tiles_per_block, p.blocks,
+                         (const unsigned*)hist, (const unsigned*)totals);
+    };
+    using Big = std::integral_constant<int, BIG_SCATTER_BLOCK>;
+    using Small = std::integral_constant<int, BLOCK>;
+    if (p.scatter_threads == BIG_SCATTER_BLOCK) {
+      if (i == 0) scatter(std::true_type{}, Big{}); else scatter(std::false_type{}, Big{});
+    } else {
+      if (i == 0) scatter(std::true_type{}, Small{}); else scatter(std::false_type{}, Small{});
+    }
+    keys_in = keys_out;
+    vals_in = vals_out;
+  }
+  return hipGetLastError();
 }
 
 // dst[k] = src[perm[k]] (gather) or dst[perm[k]] = src[k] (scatter) for rows of `vecs` vectors of type T.
@@ -248,15 +604,8 @@ int flexspmv_coo_rows_to_csr(const void* row_ids, int index_bytes, int64_t ne, i
 }
 
 size_t flexspmv_sort_workspace_bytes(int64_t ne, int64_t num_rows) {
-  if (ne <= 0 || ne >= ((int64_t)1 << 31) || num_rows <= 0) return 0;
-  size_t bytes = 0;
-  // the key iterator's type does not change the scratch layout; the wider index type is queried
-  if (sort_pairs<int64_t>(nullptr, bytes, (const int64_t*)nullptr, nullptr, nullptr, ne, num_rows, nullptr) != hipSuccess)
-    return 0;
-  size_t bytes32 = 0;
-  if (sort_pairs<int32_t>(nullptr, bytes32, (const int32_t*)nullptr, nullptr, nullptr, ne, num_rows, nullptr) != hipSuccess)
-    return 0;
-  return bytes > bytes32 ? bytes : bytes32;
+  if (ne <= 0 || ne >= ((int64_t)1 << 31) || num_rows <= 0 || num_rows >= ((int64_t)1 << 31)) return 0;
+  return plan_sort(ne, num_rows).bytes;
 }
 
 int flexspmv_sort_edges_by_row(const void* row_ids, int index_bytes, int64_t ne, int64_t num_rows,
@@ -270,17 +619,18 @@ int flexspmv_sort_edges_by_row(const void* row_ids, int index_bytes, int64_t ne,
     return fail(FLEXSPMV_FORMATS_ERR_BAD_ARGUMENT, "a pointer is NULL");
   if (ne >= ((int64_t)1 << 31) || num_rows >= ((int64_t)1 << 31))
     return fail(FLEXSPMV_FORMATS_ERR_TOO_LARGE, "ne and num_rows must stay below 2^31 (32-bit offsets)");
-  const size_t need = flexspmv_sort_workspace_bytes(ne, num_rows);
-  if (need > 0 && (workspace == nullptr || workspace_bytes < need))
+  const SortPlan plan = plan_sort(ne, num_rows);
+  if (workspace == nullptr || workspace_bytes < plan.bytes)
     return fail(FLEXSPMV_FORMATS_ERR_WORKSPACE, "workspace is missing or smaller than flexspmv_sort_workspace_bytes()");
-  size_t bytes = workspace_bytes;
+  if (((uintptr_t)workspace & 3u) != 0)
+    return fail(FLEXSPMV_FORMATS_ERR_BAD_ARGUMENT, "workspace must be aligned to 4 bytes");
   const hipError_t e =
       index_bytes == 4
-          ? sort_pairs<int32_t>(workspace, bytes, (const int32_t*)row_ids, sorted_rows, permutation, ne, num_rows,
+          ? sort_pairs<int32_t>(plan, workspace, (const int32_t*)row_ids, sorted_rows, permutation, ne, num_rows,
                                 (hipStream_t)stream)
-          : sort_pairs<int64_t>(workspace, bytes, (const int64_t*)row_ids, sorted_rows, permutation, ne, num_rows,
+          : sort_pairs<int64_t>(plan, workspace, (const int64_t*)row_ids, sorted_rows, permutation, ne, num_rows,
                                 (hipStream_t)stream);
-  if (e != hipSuccess) return fail_hip(e, "radix sort failed");
+  if (e != hipSuccess) return fail_hip(e, "kernel launch failed");
   return FLEXSPMV_FORMATS_OK;
 }
 

@@ -64,6 +64,25 @@ struct Tensor {
 #pragma unroll
     for (int i = 0; i < N; ++i) values[i] = src[i];
   }
+  // Vertex data addressed through an index (second memory level).
+  static FLEX_DEV Tensor gathered(const V* src) {
+#ifdef FLEX_TUNE_GATHER_POLICY
+    Tensor t;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+#if FLEX_TUNE_GATHER_POLICY == 1
+      t.values[i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#elif FLEX_TUNE_GATHER_POLICY == 2
+      t.values[i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+#else
+      t.values[i] = __builtin_nontemporal_load(src + i);
+#endif
+    }
+    return t;
+#else
+    return Tensor(src);
+#endif
+  }
   FLEX_DEV V& operator[](int i) { return values[i]; }
   FLEX_DEV const V& operator[](int i) const { return values[i]; }
   FLEX_DEV Tensor& operator=(V fill) {

@@ -54,14 +54,21 @@ enum flexspmv_formats_status {
 int flexspmv_coo_rows_to_csr(const void* row_ids, int index_bytes, int64_t ne, int64_t num_rows,
                              int32_t* row_ptr, int32_t* findings, void* stream);
 
-/* Scratch bytes flexspmv_sort_edges_by_row needs. */
+/* Scratch bytes flexspmv_sort_edges_by_row needs: per-block digit counters, and a second pair of
+ * int32[ne] buffers when the ids need more than one 8-bit digit (num_rows > 256).  0 when ne == 0 or a
+ * size is out of range. */
 size_t flexspmv_sort_workspace_bytes(int64_t ne, int64_t num_rows);
 
-/* Stable sort of the edges by row id.
+/* Stable sort of the edges by row id (radix sort over the bits num_rows - 1 needs; kernels of this
+ * library only: it clears nothing, allocates nothing and may be captured into a HIP graph).
  *   sorted_rows   int32[ne]: the row ids in ascending order
  *   permutation   int32[ne]: permutation[k] = position in the original list of the edge now at k
- * Row ids must lie in [0, num_rows); ids outside are reported through flexspmv_coo_rows_to_csr on
- * sorted_rows.  ne == 0 is allowed. */
+ *   workspace     flexspmv_sort_workspace_bytes(ne, num_rows) bytes, 4-byte aligned; must not overlap
+ *                 row_ids, sorted_rows or permutation
+ * Row ids must lie in [0, num_rows).  An id outside is ordered as if it were num_rows - 1 (it stays in
+ * its original order among that row's edges), keeps its value in sorted_rows (-1 if it does not fit an
+ * int32) and is reported by flexspmv_coo_rows_to_csr on sorted_rows.  row_ids may alias neither output.
+ * ne == 0 is allowed. */
 int flexspmv_sort_edges_by_row(const void* row_ids, int index_bytes, int64_t ne, int64_t num_rows,
                                int32_t* sorted_rows, int32_t* permutation, void* workspace,
                                size_t workspace_bytes, void* stream);

@@ -122,10 +122,28 @@ def test_bad_arguments_are_refused_before_any_device_work():
     assert lib.flexspmv_sort_edges_by_row(p, 4, 5, 0, p, p, p, 1 << 20, None) == -1
     assert lib.flexspmv_sort_edges_by_row(None, 4, 5, 10, p, p, p, 1 << 20, None) == -1
     assert lib.flexspmv_sort_edges_by_row(p, 4, 0, 10, p, p, None, 0, None) == 0       # nothing to sort
+    need = lib.flexspmv_sort_workspace_bytes(5, 10)
+    assert need > 0
+    assert lib.flexspmv_sort_edges_by_row(p, 4, 5, 10, p, p, p, need - 1, None) == -4   # scratch too small
+    assert b"workspace" in lib.flexspmv_formats_last_error()
+    assert lib.flexspmv_sort_edges_by_row(p, 4, 5, 10, p, p, None, need, None) == -4
     assert lib.flexspmv_gather_rows(p, p, p, 5, 6, None) == -1                           # not a multiple of 4
     assert lib.flexspmv_gather_rows(p, p, None, 5, 8, None) == -1
     assert lib.flexspmv_scatter_rows(p, p, p, -1, 8, None) == -1
     assert lib.flexspmv_scatter_rows(p, p, p, 0, 8, None) == 0
+
+
+def test_sort_scratch_follows_the_number_of_digits():
+    """One 8-bit digit: counters only.  More digits: a second pair of buffers of ne words each as well."""
+    lib = _lib()
+    one_digit = lib.flexspmv_sort_workspace_bytes(100_000, 256)
+    two_digits = lib.flexspmv_sort_workspace_bytes(100_000, 257)
+    four_digits = lib.flexspmv_sort_workspace_bytes(100_000, 2 ** 31 - 1)
+    assert 0 < one_digit < 100_000                      # 256 counters per block of 16 384 ids, 256 sums
+    assert two_digits >= one_digit + 2 * 4 * 100_000
+    assert four_digits == two_digits                    # the two pairs of buffers alternate
+    assert lib.flexspmv_sort_workspace_bytes(0, 10) == 0
+    assert lib.flexspmv_sort_workspace_bytes(2 ** 31, 10) == 0
 
 
 def test_host_side_refuses_cpu_tensors():
@@ -222,6 +240,118 @@ def test_sort_then_row_pointer_reports_out_of_range_ids():
     sorted_rows, _ = formats.sort_edges_by_row(torch.from_numpy(rows).cuda(), 10)
     with pytest.raises(RuntimeError, match="outside"):
         formats.coo_rows_to_csr(sorted_rows, 10)
+
+
+@pytest.mark.gpu
+def test_sort_at_tile_boundaries_and_digit_counts():
+    """Lengths around one, two and four 4 096-pair tiles (what lists below 16 M pairs are cut into) and row counts
+    whose ids need 1 ... 4 digits (8, 9, 16, 17, 24, 25, 31 bits): sorted ids and permutation equal numpy's stable sort."""
+    torch = _cuda()
+    rng = np.random.default_rng(17)
+    sizes = [1, 63, 64, 65, 4095, 4096, 4097, 16383, 16384, 16385, 32767, 32768, 32769, 100_003]
+    for ne in sizes:
+        for num_rows in (1, 2, 255, 256, 257, 65536, 65537, (1 << 24), (1 << 24) + 1, (1 << 31) - 1):
+            rows = rng.integers(0, num_rows, ne).astype(np.int64)
+            rows[rng.integers(0, ne, max(1, ne // 7))] = num_rows - 1          # the last row is always there
+            print(f"case ne={ne} rows={num_rows}", flush=True)
+            exp_rows, exp_perm = FO.sort_edges_by_row(rows)
+            got_rows, got_perm = formats.sort_edges_by_row(torch.from_numpy(rows).cuda(), num_rows)
+            assert np.array_equal(got_rows.cpu().numpy(), exp_rows)
+            assert np.array_equal(got_perm.cpu().numpy(), exp_perm)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("extra", [0, 1, 16383, 16384 + 5])
+def test_sort_of_long_lists_at_tile_boundaries(extra):
+    """From 16 M pairs on the scatter works on tiles of 16 384 pairs (1024 threads): lengths at and around a tile end."""
+    torch = _cuda()
+    rng = np.random.default_rng(19 + extra)
+    ne, num_rows = (16 << 20) + extra, 3_000_001
+    rows = rng.integers(0, num_rows, ne).astype(np.int32)
+    exp_rows, exp_perm = FO.sort_edges_by_row(rows)
+    got_rows, got_perm = formats.sort_edges_by_row(torch.from_numpy(rows).cuda(), num_rows)
+    assert np.array_equal(got_rows.cpu().numpy(), exp_rows)
+    assert np.array_equal(got_perm.cpu().numpy(), exp_perm)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("index_dtype", ["int32", "int64"])
+def test_sort_of_ids_that_are_not_16_byte_aligned(index_dtype):
+    torch = _cuda()
+    rng = np.random.default_rng(23)
+    for skip in (1, 2, 3):
+        rows = rng.integers(0, 5000, 70_001).astype(index_dtype)
+        padded = torch.from_numpy(np.concatenate([np.zeros(skip, index_dtype), rows])).cuda()
+        exp_rows, exp_perm = FO.sort_edges_by_row(rows)
+        got_rows, got_perm = formats.sort_edges_by_row(padded[skip:], 5000)
+        assert np.array_equal(got_rows.cpu().numpy(), exp_rows)
+        assert np.array_equal(got_perm.cpu().numpy(), exp_perm)
+
+
+@pytest.mark.gpu
+def test_sort_keeps_ids_outside_the_rows_in_place_among_the_last_row():
+    """Ids outside [0, num_rows) sort as the last row (in original order among its edges) and keep their value,
+    -1 if it does not fit an int32; nothing else moves."""
+    torch = _cuda()
+    rows = np.array([5, 9, 1, 12, 9, -3, 3, 2 ** 40, 9, 0], dtype=np.int64)
+    sorted_rows, perm = formats.sort_edges_by_row(torch.from_numpy(rows).cuda(), 10)
+    assert sorted_rows.cpu().tolist() == [0, 1, 3, 5, 9, 12, 9, -1, -1, 9]
+    assert perm.cpu().tolist() == [9, 2, 6, 0, 1, 3, 4, 5, 7, 8]
+
+
+@pytest.mark.gpu
+def test_sort_with_several_tiles_per_block_matches_torch():
+    """Poisson-sized list (117 M ids, 16.8 M rows): more than 4096 tiles, so every scatter block walks two tiles
+    and carries its digit offsets from one to the next.  torch's stable sort is the second opinion."""
+    torch = _cuda()
+    ne, num_rows = 117_047_296, 16_777_216
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    rows = torch.randint(0, num_rows, (ne,), device="cuda", dtype=torch.int32, generator=gen)
+    sorted_rows, perm = formats.sort_edges_by_row(rows, num_rows)
+    ref_rows, ref_perm = torch.sort(rows, stable=True)
+    assert torch.equal(sorted_rows, ref_rows)
+    assert torch.equal(perm, ref_perm.to(torch.int32))
+
+
+@pytest.mark.gpu
+def test_sort_replays_in_a_hip_graph():
+    """The sort clears nothing and allocates nothing: captured once, replayed on new ids in the same buffers
+    (eager sorts and synchronisation between the replays), every replay equals the oracle."""
+    torch = _cuda()
+    rng = np.random.default_rng(37)
+    num_rows, ne = 50_000, 200_000
+    lib = formats.library()
+    ids = torch.zeros(ne, dtype=torch.int32, device="cuda")
+    out_rows = torch.empty(ne, dtype=torch.int32, device="cuda")
+    out_perm = torch.empty(ne, dtype=torch.int32, device="cuda")
+    need = lib.flexspmv_sort_workspace_bytes(ne, num_rows)
+    workspace = torch.empty(need, dtype=torch.uint8, device="cuda")
+
+    def sort_into_buffers():
+        stream = torch.cuda.current_stream().cuda_stream
+        assert lib.flexspmv_sort_edges_by_row(ids.data_ptr(), 4, ne, num_rows, out_rows.data_ptr(), out_perm.data_ptr(),
+                                              workspace.data_ptr(), need, stream) == 0
+
+    ids.copy_(torch.from_numpy(_edge_list(rng, num_rows, ne, "uniform").astype(np.int32)))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        sort_into_buffers()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sort_into_buffers()
+    for rep, kind in enumerate(["skewed", "few_rows", "uniform", "tail"]):
+        rows = rng.permutation(_edge_list(rng, num_rows, ne, kind)).astype(np.int32)
+        ids.copy_(torch.from_numpy(rows))
+        graph.replay()
+        torch.cuda.synchronize()
+        exp_rows, exp_perm = FO.sort_edges_by_row(rows)
+        assert np.array_equal(out_rows.cpu().numpy(), exp_rows), (rep, kind)
+        assert np.array_equal(out_perm.cpu().numpy(), exp_perm), (rep, kind)
+        eager_rows, eager_perm = formats.sort_edges_by_row(ids, num_rows)     # eager work between replays
+        assert torch.equal(eager_rows, out_rows) and torch.equal(eager_perm, out_perm)
 
 
 @pytest.mark.gpu

@@ -107,12 +107,11 @@ def test_generated_source_is_deterministic_and_hash_keyed():
 
 
 def test_no_cuda_or_compat_layers_in_kernel_sources():
+    """Every kernel is this package's own: no CUB / hipCUB / rocPRIM primitive, no dual-platform switch."""
     bad = re.compile(r"cub::|hipcub|rocprim|__HIP_PLATFORM|cuda_runtime|triton", re.I)
-    # the set-up-time sort of an unordered edge list is rocPRIM's radix sort; nothing on the launch path is
-    sort_only = re.compile(r"cub::|hipcub|__HIP_PLATFORM|cuda_runtime|triton", re.I)
     for fn in os.listdir(build.CSRC_DIR):
         with open(os.path.join(build.CSRC_DIR, fn)) as f:
-            assert not (sort_only if fn == "flex_formats.hip" else bad).search(f.read()), fn
+            assert not bad.search(f.read()), fn
 
 
 # ---------------------------------------------------------------------------------------------
