@@ -149,7 +149,7 @@ rows_search_kernel(const I* __restrict__ rows, const int ne, const int num_rows,
 //   sort_scan_kernel        block d turns row d of hist into exclusive prefixes and leaves the row's sum
 //   sort_scatter_kernel     block b ranks its tiles' items (wave64 ballots give every item the lanes that
 //                           hold the same digit; wavefront counters in LDS carry the order across the 16
-//                           items of a lane and across the 4 wavefronts), orders a tile by digit in LDS
+//                           items of a lane and across the block's wavefronts), orders a tile by digit in LDS
 //                           and writes each digit's run to its place: neighbouring lanes write
 //                           neighbouring words.
 // Position order inside a tile is wavefront-major: item k of lane l of wavefront w is element
