@@ -167,6 +167,19 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
 
+    # A region of K launches of a small workload is over in a millisecond and one hiccup of the host doubles
+    # it: such a workload gets six more regions of K launches each, and the median of the seven is reported
+    # beside the first.
+    region_ms = [ms_per_step]
+    if ms_per_step * steps < 10.0:
+        for _ in range(6):
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                ext.merged_spmv_launch(*args)
+            torch.cuda.synchronize()
+            region_ms.append((time.perf_counter() - t0) * 1e3 / steps)
+    region_ms.sort()
+
     # the same launches one by one, each between two events on the launch stream
     step_ms = []
     for _ in range(steps):
@@ -178,8 +191,36 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
         step_ms.append(e0.elapsed_time(e1))
     step_ms.sort()
 
-    # the same with the tile table kept between launches (legitimate when the sparsity pattern is
-    # fixed, as in a solver loop); reported beside the headline, never as the headline
+    # Where the blocks of a launch take their tile boundaries from is a policy of the library (flexspmv.h: the tile
+    # table): most launches try the table the launch before left in their scratch and confirm it, block by block,
+    # against the row pointer they are given - the timed region above follows the warm-up on the same matrix, so
+    # its blocks confirm and no search runs -, large launches with row-snapped tiles run a search kernel first.
+    # Beside the default, the same K launches with every boundary searched afresh on every launch, as the
+    # reference does, with the table confirmed ...
+    ms_per_step_search = ms_per_step_confirm = None
+    default_source = None
+    if ext.signature["has_reducer"]:
+        from flexspmv_amd.binding import DTYPE_CODES, FLAG_CONFIRM_TILES, FLAG_SEARCH_TILES
+        import ctypes
+        shape = (ctypes.c_int32 * 6)()
+        ext._lib.flexspmv_tiling(DTYPE_CODES[str(next(iter(w.tensors.values())).dtype)], int(w.num_rows), int(w.ne), shape)
+        default_source = "table confirmed in the blocks" if shape[5] == 1 or shape[2] == 0 else "search kernel"
+
+        def with_flag(flag):
+            ext.extra_flags |= flag
+            warm_up()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                o = ext.merged_spmv_launch(*args)
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) * 1e3 / steps
+            ext.extra_flags &= ~flag
+            for x, y in zip(outs, o):
+                assert torch.equal(x, y), "the source of the tile boundaries changed the result"
+            return ms
+        ms_per_step_search = with_flag(FLAG_SEARCH_TILES)
+        ms_per_step_confirm = with_flag(FLAG_CONFIRM_TILES)
+    # ... and with the table taken on the caller's word, without the confirmation
     ms_per_step_reuse = None
     if ext.signature["has_reducer"]:
         ext.reuse_tiles = True
@@ -219,6 +260,8 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
         "workload": w.name, "graph": w.graph, "dtype": dtype,
         "ne": int(w.ne), "num_rows": int(w.num_rows), "algorithmic_bytes": int(w.algorithmic_bytes),
         "flops": int(w.flops), "ms_per_step": ms_per_step,
+        **({"ms_per_step_median_of_regions": region_ms[len(region_ms) // 2], "regions": len(region_ms)}
+           if len(region_ms) > 1 else {}),
         "step_ms_median": step_ms[len(step_ms) // 2], "step_ms_min": step_ms[0],
         "kernel": "flex::flat_kernel" if flat else "flex::reduce_kernel",
         "kernel_ms": kernel_ms_mean, "kernel_ms_median": kernel_ms[len(kernel_ms) // 2], "kernel_ms_min": kernel_ms[0],
@@ -232,6 +275,12 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
         result["library_variant"] = ext.variant   # tuning switches and tile-shape override the file was built with
     if machine:
         result["machine"] = machine
+    if ms_per_step_search is not None:
+        result["tile_boundaries_by_default"] = default_source
+        result["ms_per_step_search_every_launch"] = ms_per_step_search
+        result["gbs_search_every_launch"] = w.algorithmic_bytes / ms_per_step_search / 1e6
+        result["ms_per_step_table_confirmed"] = ms_per_step_confirm
+        result["gbs_table_confirmed"] = w.algorithmic_bytes / ms_per_step_confirm / 1e6
     if ms_per_step_reuse is not None:
         result["ms_per_step_tile_reuse"] = ms_per_step_reuse
         result["gbs_tile_reuse"] = w.algorithmic_bytes / ms_per_step_reuse / 1e6
@@ -461,7 +510,10 @@ def main() -> int:
     for name, wo, r, o in pending:
         r = cpu_leg(wo, r, o, min(a.cpu_runs, 3))
         entry = {k: r[k] for k in ("workload", "graph", "dtype", "ne", "num_rows", "algorithmic_bytes", "seed", "policy",
-                                   "ms_per_step", "step_ms_median", "step_ms_min", "gbs", "edges_per_s", "gflops",
+                                   "ms_per_step", "ms_per_step_median_of_regions", "regions", "step_ms_median",
+                                   "step_ms_min", "gbs", "edges_per_s", "gflops",
+                                   "tile_boundaries_by_default", "ms_per_step_search_every_launch",
+                                   "gbs_search_every_launch", "ms_per_step_table_confirmed", "gbs_table_confirmed",
                                    "ms_per_step_tile_reuse", "gbs_tile_reuse") if k in r}
         entry["pct_of_hbm_peak"] = 100.0 * r["gbs"] / HBM_PEAK_GBS
         entry["roofline"] = roofline_of(r)
@@ -491,6 +543,7 @@ def main() -> int:
                                + f" ({head['graph']})", "ne": head["ne"],
                    "num_rows": head["num_rows"], "algorithmic_bytes": head["algorithmic_bytes"],
                    "policy": head["policy"], "seed": head["seed"]},
+        **({k: head[k] for k in ("ms_per_step_median_of_regions", "regions") if k in head}),
         "step_ms_median": head["step_ms_median"],
         "step_ms_min": head["step_ms_min"],
         "pct_of_hbm_peak": 100.0 * head["gbs"] / HBM_PEAK_GBS,
@@ -504,10 +557,22 @@ def main() -> int:
     if a.library:
         line["config"]["library"] = a.library   # not the shipped library: a variant built for a measurement
         line["config"]["library_variant"] = head["library_variant"]
-    if "ms_per_step_tile_reuse" in head:
-        line["with_tile_reuse"] = {"ms_per_step": head["ms_per_step_tile_reuse"], "value": head["gbs_tile_reuse"],
-                                   "unit": "GB/s", "note": "tile table of the previous launch reused "
-                                   "(FLEXSPMV_FLAG_REUSE_TILES); the headline value recomputes it every step"}
+    if "ms_per_step_search_every_launch" in head:
+        line["tile_table"] = {
+            "headline": head["tile_boundaries_by_default"] + " (the library's default for this launch; flexspmv.h, the "
+                        "tile table)",
+            "search_every_launch": {"ms_per_step": head["ms_per_step_search_every_launch"],
+                                    "value": head["gbs_search_every_launch"], "unit": "GB/s",
+                                    "note": "FLEXSPMV_FLAG_SEARCH_TILES: every boundary searched on every launch, as the "
+                                            "reference does"},
+            "table_confirmed": {"ms_per_step": head["ms_per_step_table_confirmed"], "value": head["gbs_table_confirmed"],
+                                "unit": "GB/s",
+                                "note": "FLEXSPMV_FLAG_CONFIRM_TILES: every block takes its boundaries from the table the "
+                                        "launch before left in the scratch and confirms them against this launch's row "
+                                        "pointer (three row ends per boundary, fetched with the tile); the timed launches "
+                                        "follow the warm-up on the same matrix, so no search runs in them"},
+            "taken_on_trust": {"ms_per_step": head["ms_per_step_tile_reuse"], "value": head["gbs_tile_reuse"],
+                               "unit": "GB/s", "note": "FLEXSPMV_FLAG_REUSE_TILES: the table used without the confirmation"}}
     if "cpu" in head:
         line["cpu_baseline"] = cpu_baseline_of(head)
     if others:

@@ -30,11 +30,13 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 from . import build as _build
 from .ir import FusedGraphIR
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 FLAG_TIME_KERNEL = 1
 FLAG_REUSE_TILES = 2
 FLAG_KEEP_TILES = 4
 FLAG_DEBUG_SYNC = 8
+FLAG_SEARCH_TILES = 16
+FLAG_CONFIRM_TILES = 32
 DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
 EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
                     "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms", "flexspmv_tiling",
@@ -161,15 +163,16 @@ class HipExtension:
         self._streamed = set(self.signature["non_gather_value_inputs"])
         self._dtypes = set(self.signature["dtypes"])
         self._param_names = [p["name"] for p in self.signature["params"]]
-        self._workspace: Dict[Any, Any] = {}   # (device index, stream handle) -> scratch tensor
+        self._workspace: Dict[Any, Any] = {}   # (device index, stream handle, row pointer address) -> scratch tensor
         self._last_used: Dict[Any, int] = {}   # ... -> number of the last launch that used it
         self._launch_count = 0
         self._captured = set()                 # keys whose buffer a stream capture has recorded
         self._retained: List[Any] = []         # replaced buffers that a captured graph still refers to
         self.time_kernel = False   # set True to bracket the dominant kernel of each launch with events
-        # Reuse of the tile table between launches on the same, unmodified row_end_offsets tensor (the
-        # reference's wrapper keeps it as an immutable buffer, dynamic_replace_submodule.py:118-137).
-        # Off by default: every launch then does all the work a launch of the reference does.
+        # Every launch tries the tile table the launch before left in its scratch and confirms it, block by
+        # block, against the row pointer it was given (the library's default).  reuse_tiles = True skips that
+        # check too on launches whose row_end_offsets tensor is the same, unmodified one as in the launch before
+        # (the reference's wrapper keeps it as an immutable buffer, dynamic_replace_submodule.py:118-137).
         self.reuse_tiles = False
         self._tile_key = None
         self.extra_flags = 0       # FLAG_* bits added to every launch (FLAG_DEBUG_SYNC: print every kernel's
@@ -205,9 +208,11 @@ class HipExtension:
     MAX_IDLE_SCRATCH = 8
     IDLE_LAUNCHES = 64
 
-    def _scratch(self, device, index: int, raw_stream: int, nbytes: int):
+    def _scratch(self, device, index: int, raw_stream: int, nbytes: int, row_ptr: int = 0):
         """Scratch of this library for launches on the stream with handle ``raw_stream`` of device ``index``
-        (the current stream of the current device when this is called).
+        (the current stream of the current device when this is called) with the row pointer at address
+        ``row_ptr``: a launch finds the tile table of the launch before in its scratch, so a caller that
+        alternates between matrices keeps one scratch - one table - per matrix.
 
         The buffer is allocated on that stream and only ever used on it, so when a larger launch replaces
         it - or when it is dropped - the caching allocator hands the old block out again in stream order:
@@ -217,7 +222,7 @@ class HipExtension:
         many streams does not grow the table without bound: beyond MAX_IDLE_SCRATCH entries, buffers of
         streams that have not launched for IDLE_LAUNCHES launches are dropped (never a captured one)."""
         import torch
-        key = (index, raw_stream)
+        key = (index, raw_stream, row_ptr)
         self._launch_count += 1
         buf = self._workspace.get(key)
         capturing = torch._C._cuda_isCurrentStreamCapturing()
@@ -247,14 +252,18 @@ class HipExtension:
                 del self._workspace[k]
                 self._last_used.pop(k, None)
 
-    def workspace_of(self, device, stream=None):
-        """The scratch tensor of launches on ``stream`` (default: the current stream) of ``device``, or
-        None before the first such launch.  For debugging (the tile table sits at its start)."""
+    def workspace_of(self, device, stream=None, row_end_offsets=None):
+        """The scratch tensor of launches on ``stream`` (default: the current stream) of ``device`` with the
+        given row pointer (default: whichever launched last on that stream), or None before the first such
+        launch.  For debugging (the tile table sits at its start)."""
         import torch
         device = torch.device(device)
         stream = stream if stream is not None else torch.cuda.current_stream(device)
         index = device.index if device.index is not None else torch.cuda.current_device()
-        return self._workspace.get((index, int(stream.cuda_stream)))
+        if row_end_offsets is not None:
+            return self._workspace.get((index, int(stream.cuda_stream), row_end_offsets.data_ptr()))
+        mine = [k for k in self._workspace if k[0] == index and k[1] == int(stream.cuda_stream)]
+        return self._workspace[max(mine, key=lambda k: self._last_used.get(k, 0))] if mine else None
 
     # -- the call ------------------------------------------------------------------------
     def _call_state(self):
@@ -424,7 +433,7 @@ class HipExtension:
         """Fill the argument block and call the library on the current stream of the (current) device."""
         import torch
         raw_stream = torch._C._cuda_getCurrentRawStream(index)
-        ws = self._scratch(device, index, raw_stream, ws_bytes)
+        ws = self._scratch(device, index, raw_stream, ws_bytes, ro.data_ptr() if self._has_reducer else 0)
         st = self._call_state()
         la = st.la
         for i, t in enumerate(values):

@@ -134,8 +134,10 @@ struct Tiling {
   int row_group;   // row path: edges of a row staged at a time (<= the kernel's register budget; 0: that budget)
 };
 
+// split: the row the search stopped at, before the boundary was moved (boundary_from_split rebuilds the
+// boundary from it).
 __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end, int num_rows,
-                                              int nnz) {
+                                              int nnz, int& split) {
   const long long d = (long long)t * tl.nominal;
   const int diag = (int)min(d, (long long)num_rows + nnz);
 #ifdef FLEX_TUNE_BISECTION_ONLY  // tuning switch: the reference's plain bisection
@@ -143,9 +145,34 @@ __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int
 #else
   int2 c = merge_path_search_interp(diag, row_end, num_rows, nnz);
 #endif
+  split = c.x;
   if (tl.snap_slack > 0 && t > 0 && t < tl.num_tiles) {
     const int xs = c.x & ~tl.snap_mask;
     const int ys = xs > 0 ? row_end[xs - 1] : 0;  // first non-zero of row xs
+    if ((c.x - xs) + (c.y - ys) <= tl.snap_slack) c = make_int2(xs, ys);
+  }
+  return c;
+}
+
+// The boundary a search on tile boundary t returns, rebuilt from a claimed split and three row ends: the one
+// of the row before the split, the one of the row at it, and the one of the row before the row a snap would
+// move the boundary to (values for rows outside the matrix are never looked at).  ok: the claim is what a
+// search finds - g(i) = row_end[i] + i + 1 is strictly increasing and the split is the first i of its
+// bracket with g(i) > diag, so its two neighbours decide.  A block that is handed the tile table of an
+// earlier launch checks it this way against the row pointer of this launch: three loads that travel with
+// the tile's own instead of a search in front of them.
+__device__ __forceinline__ int2 boundary_from_split(int t, const Tiling& tl, int num_rows, int nnz, int split,
+                                                    int end_before, int end_at, int end_before_snap_row, bool& ok) {
+  const long long d = (long long)t * tl.nominal;
+  const int diag = (int)min(d, (long long)num_rows + nnz);
+  const int lo = max(diag - nnz, 0);
+  const int hi = min(diag, num_rows);
+  ok = split >= lo && split <= hi && (split == hi || end_at + split + 1 > diag) &&
+       (split == lo || end_before + split <= diag);
+  int2 c = make_int2(split, diag - split);
+  if (tl.snap_slack > 0 && t > 0 && t < tl.num_tiles) {
+    const int xs = split & ~tl.snap_mask;
+    const int ys = xs > 0 ? end_before_snap_row : 0;
     if ((c.x - xs) + (c.y - ys) <= tl.snap_slack) c = make_int2(xs, ys);
   }
   return c;
@@ -163,7 +190,7 @@ __device__ __forceinline__ int2 tile_boundary(int t, const Tiling& tl, const int
 // tile_boundary (same monotone predicate, same rule).
 template <int W>
 __device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end,
-                                                    int num_rows, int nnz) {
+                                                    int num_rows, int nnz, int& split) {
   static_assert(W == 2 || W == 4 || W == 8 || W == 16 || W == 32 || W == 64, "group width");
   constexpr int LEAD = (W * 5) / 8;  // rows of the window below the guess (towards the row a snap moves back to)
   const int lane = lane_id();
@@ -260,6 +287,7 @@ __device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, con
     hi = new_hi;
   }
   int2 c = make_int2(min(lo, num_rows), diag - lo);
+  split = c.x;
   if (snapping) {
     const int xs = c.x & ~tl.snap_mask;
     int ys = 0;
@@ -281,10 +309,11 @@ __device__ __forceinline__ int2 group_tile_boundary(int t, const Tiling& tl, con
 
 // ... by a whole wavefront: the result is uniform, which the compiler is told
 __device__ __forceinline__ int2 wave_tile_boundary(int t, const Tiling& tl, const int* __restrict__ row_end,
-                                                   int num_rows, int nnz) {
-  int2 c = group_tile_boundary<WAVE>(t, tl, row_end, num_rows, nnz);
+                                                   int num_rows, int nnz, int& split) {
+  int2 c = group_tile_boundary<WAVE>(t, tl, row_end, num_rows, nnz, split);
   c.x = __builtin_amdgcn_readfirstlane(c.x);
   c.y = __builtin_amdgcn_readfirstlane(c.y);
+  split = __builtin_amdgcn_readfirstlane(split);
   return c;
 }
 
@@ -303,14 +332,22 @@ constexpr int SEARCH_BLOCK = FLEX_TUNE_SEARCH_BLOCK;
 #endif
 constexpr int SEARCH_GROUP = FLEX_TUNE_SEARCH_GROUP;
 __global__ void __launch_bounds__(SEARCH_BLOCK)
-tile_search_kernel(const Tiling tl, const int* __restrict__ row_end, int num_rows, int nnz, int2* __restrict__ coords) {
+tile_search_kernel(const Tiling tl, const int* __restrict__ row_end, int num_rows, int nnz, int2* __restrict__ coords,
+                   int* __restrict__ splits) {
   const int t = (int)(blockIdx.x * (SEARCH_BLOCK / SEARCH_GROUP) + threadIdx.x / SEARCH_GROUP);
   if (t > tl.num_tiles) return;  // uniform per group
+  int split;
 #ifdef FLEX_TUNE_THREAD_SEARCH  // tuning switch: one lane searches
-  if ((threadIdx.x & (SEARCH_GROUP - 1)) == 0) coords[t] = tile_boundary(t, tl, row_end, num_rows, nnz);
+  if ((threadIdx.x & (SEARCH_GROUP - 1)) == 0) {
+    coords[t] = tile_boundary(t, tl, row_end, num_rows, nnz, split);
+    splits[t] = split;
+  }
 #else
-  const int2 c = group_tile_boundary<SEARCH_GROUP>(t, tl, row_end, num_rows, nnz);
-  if ((threadIdx.x & (SEARCH_GROUP - 1)) == 0) coords[t] = c;
+  const int2 c = group_tile_boundary<SEARCH_GROUP>(t, tl, row_end, num_rows, nnz, split);
+  if ((threadIdx.x & (SEARCH_GROUP - 1)) == 0) {
+    coords[t] = c;
+    splits[t] = split;
+  }
 #endif
 }
 
@@ -371,11 +408,19 @@ constexpr int edges_per_load() {
 // lanes read a clamped address, and per-item work is predicated.  Every row is written exactly once;
 // the tile's open last row becomes a carry record for fixup_kernel.
 // ----------------------------------------------------------------------------------------------
+//
+// check (uniform): c0 and c1 come from the tile table of an earlier launch, together with the splits they
+// were derived from.  Six lanes then fetch the row ends that decide whether a search on this launch's row
+// pointer would return the same two boundaries (boundary_from_split); the loads travel with the tile's own,
+// the verdict is part of the vote, and a tile whose boundaries are not confirmed returns true before
+// anything has been written: its block searches and comes back.
 template <class G, int BLOCK, int IPT, int EPL>
-__device__ __forceinline__ void
-reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hint, const int num_rows,
-            const int* __restrict__ row_end, const int nnz, const typename G::Params& p, int* __restrict__ carry_row,
-            typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials) {
+__device__ __forceinline__ bool
+reduce_tile(const int tile, const int2 c0, const int2 c1, const Tiling& tl, const bool check, const int split0,
+            const int split1, const int num_rows, const int* __restrict__ row_end, const int nnz,
+            const typename G::Params& p, int* __restrict__ carry_row, typename G::Value* __restrict__ carry_val,
+            typename G::Value* __restrict__ agg_partials) {
+  const int row_group_hint = tl.row_group;
   using V = typename G::Value;
   using Fetch = typename G::Fetch;
   using Gather = typename G::Gather;
@@ -433,7 +478,12 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   __shared__ int s_wave_key[NW];
   __shared__ V s_wave_val[NW][REDN];
 
-  const int tid = threadIdx.x;
+  // The thread id is taken afresh on every call: a kernel holds this function twice (a tile taken from the
+  // table, and the same tile again after a search when the table was refused), and the compiler would
+  // otherwise share everything that only depends on the thread id between the two and keep it in
+  // registers through the whole first tile.
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
   const int lane = tid & (WAVE - 1);
   const int wave = tid / WAVE;
 
@@ -447,6 +497,25 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   // loads of them merge into wider ones: 16 bytes per lane instead of 4 or 8), threads side by side.
   static_assert(EPL >= 1 && IPT % EPL == 0, "edges per load must divide the items per thread");
   auto slot_of = [&](const int k) { return (k / EPL) * (EPL * BLOCK) + tid * EPL + (k % EPL); };
+
+  // 0: for a tile table that has to be confirmed, the three row ends that decide a boundary (the rows before
+  // and at the split, and the row before the one a snap moves the boundary to): lanes 0-2 of the first
+  // wavefront fetch them for the tile's start, lanes 0-2 of the second for its end (a block of one wavefront:
+  // lanes 0-2 and 3-5).  Issued in front of the tile's loads, they are back first, and the verdict is worked
+  // out while the tile's data are on the way.
+  constexpr int CHECKERS = NW >= 2 ? 2 : 1;  // wavefronts that check a boundary
+  const int wave_uniform = __builtin_amdgcn_readfirstlane(wave);  // the same number, known to be one per wavefront
+  const bool checker = check && wave_uniform < CHECKERS;
+  int check_value = 0;
+  if (checker) {
+    // which of the three rows a lane fetches, without branches: a handful of instructions in front of the
+    // tile's loads (lanes past the ones that count repeat the last row)
+    const bool of_end = CHECKERS == 2 ? wave_uniform == 1 : lane >= 3;
+    const int split = of_end ? split1 : split0;
+    const int part = min(CHECKERS == 2 || lane < 3 ? lane : lane - 3, 2);
+    const int row = (part == 2 ? (split & ~tl.snap_mask) : split) - (part != 1 ? 1 : 0);
+    check_value = row_end[min(max(row, 0), num_rows - 1)];
+  }
 
   // 1: first-level loads.  A tile holds Z <= TILE non-zeros; lanes past Z re-read the tile's last
   // edge (one cache line, no extra traffic) instead of running into the next tile's edges.
@@ -536,6 +605,30 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
     }
   }
 
+  int stale_bit = 0;
+  if (checker) {  // are the boundaries this tile is being loaded with the ones a search would find?
+    bool confirmed;
+    if constexpr (CHECKERS == 2) {
+      bool ok;
+      const int2 n = boundary_from_split(tile + wave_uniform, tl, num_rows, nnz, wave_uniform == 0 ? split0 : split1,
+                                         __builtin_amdgcn_readlane(check_value, 0),
+                                         __builtin_amdgcn_readlane(check_value, 1),
+                                         __builtin_amdgcn_readlane(check_value, 2), ok);
+      const int2 c = wave_uniform == 0 ? c0 : c1;
+      confirmed = ok && n.x == c.x && n.y == c.y;
+    } else {
+      bool ok0, ok1;
+      const int2 n0 = boundary_from_split(tile, tl, num_rows, nnz, split0, __builtin_amdgcn_readlane(check_value, 0),
+                                          __builtin_amdgcn_readlane(check_value, 1),
+                                          __builtin_amdgcn_readlane(check_value, 2), ok0);
+      const int2 n1 = boundary_from_split(tile + 1, tl, num_rows, nnz, split1, __builtin_amdgcn_readlane(check_value, 3),
+                                          __builtin_amdgcn_readlane(check_value, 4),
+                                          __builtin_amdgcn_readlane(check_value, 5), ok1);
+      confirmed = ok0 && ok1 && n0.x == c0.x && n0.y == c0.y && n1.x == c1.x && n1.y == c1.y;
+    }
+    stale_bit = confirmed ? 0 : 2;
+  }
+
   if (tid < NWORDS) s_bits[tid] = 0u;
 
   // 2: hand-over through LDS, in coalesced order.  Every slot of the tile is written (slots past Z hold
@@ -582,15 +675,17 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
   const bool my_vote = (longest > ROW_PATH_MAX_LEN) | !few_rows | uneven;
   // the ballot is taken by the whole wavefront (inside a branch it would only see the branch's lanes)
   const unsigned long long wave_votes = __builtin_amdgcn_ballot_w64(my_vote);
-  if (lane == 0) s_vote[wave] = (wave_votes != 0ull) ? 1 : 0;
+  const int vote_bits = ((wave_votes != 0ull) ? 1 : 0) | stale_bit;
+  if (lane == 0) s_vote[wave] = vote_bits;
   __syncthreads();
   int any_vote = 0;
 #pragma unroll
   for (int w = 0; w < NW; ++w) any_vote |= s_vote[w];
+  if ((any_vote & 2) != 0) return true;  // uniform: nothing has left the block yet
 #ifdef FLEX_TUNE_FORCE_MERGE  // tuning switch: always the merge path, decided at run time (same code)
-  const bool irregular = any_vote != 0 || nnz > 0;
+  const bool irregular = (any_vote & 1) != 0 || nnz > 0;
 #else
-  const bool irregular = any_vote != 0;
+  const bool irregular = (any_vote & 1) != 0;
 #endif
 
   Pack<V, AGG> agg;
@@ -885,23 +980,38 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const int row_group_hi
     }
 #endif
   }
+  return false;
 }
 
-// One block per tile.  The tile's coordinates come from the table tile_search_kernel wrote (coords !=
-// NULL), or - small launches, where a kernel of its own for the search costs more than the search -
-// from the block itself: its first two wavefronts search the two diagonals that bound the tile (the
-// reference lets two threads do it when its grid is smaller than the device, cuda_template/reducer/merged_spmv_template.cuh:97-119,
-// merged_agent_spmv_template.cuh:412-435).  coords_out != NULL makes such a block leave its
-// coordinates in the table all the same (a debugging aid: the table can then be read back).
+// Where a reducer block takes its tile's two boundaries from.
+enum TileSource : int {
+  TILES_FROM_TABLE = 0,   // the table holds this launch's boundaries (tile_search_kernel ran, or the caller
+                          // vouches for the table of an earlier launch): taken as they are
+  TILES_CONFIRMED = 1,    // the table may hold an earlier launch's boundaries, or anything else: taken if
+                          // this launch's row pointer confirms them (reduce_tile), searched otherwise
+  TILES_SEARCHED = 2      // the block searches
+};
+
+// One block per tile.  A block that searches does so with its first two wavefronts, one boundary each, on
+// the two diagonals that bound the tile (the reference lets two threads do it when its grid is smaller than
+// the device, cuda_template/reducer/merged_spmv_template.cuh:97-119, merged_agent_spmv_template.cuh:412-435)
+// and leaves boundary and split in the table, where the next launch on the same scratch finds them.
+// The default, TILES_CONFIRMED, makes the search a once-per-matrix cost without a promise from the caller:
+// a solver loop or a time stepper launches on one row structure again and again, its blocks read the
+// boundaries of the launch before, load their tiles, and the three row ends per boundary that prove the
+// boundaries right arrive with the tile's data (Poisson 256^3: no 9 us search kernel in front of the
+// reducer; spring-mass 100^3: no 3 us of search in front of every block's loads).  Table entries are only
+// ever used after this proof or after a search, whatever the scratch held: garbage, the table of another
+// matrix, or entries another block of this launch is replacing at the same moment.
 // With FLEX_TUNE_PERSISTENT (tuning switch) a launch has at most that many blocks per CU; each walks
 // tiles blockIdx.x, blockIdx.x + gridDim.x, ... and reads the coordinates of its next tile while it
 // works on the current one.
 template <class G, int BLOCK, int IPT, int EPL>
 __global__ void __launch_bounds__(BLOCK)
-reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_rows, const int* __restrict__ row_end,
-              const int nnz, const typename G::Params p, int* __restrict__ carry_row,
+reduce_kernel(int2* coords, int* splits, const int source, const Tiling tl, const int num_rows,
+              const int* __restrict__ row_end, const int nnz, const typename G::Params p, int* __restrict__ carry_row,
               typename G::Value* __restrict__ carry_val, typename G::Value* __restrict__ agg_partials,
-              int2* __restrict__ coords_out, unsigned* __restrict__ ticket) {
+              unsigned* __restrict__ ticket) {
   const int num_tiles = tl.num_tiles;
 #ifdef FLEX_TUNE_TICKET_SUM
   if (blockIdx.x == 0 && threadIdx.x == 0) *ticket = 0u;  // arms the last-block detection of fixup_kernel
@@ -918,7 +1028,7 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
       n0 = coords[next];
       n1 = coords[next + 1];
     }
-    reduce_tile<G, BLOCK, IPT, EPL>(tile, c0, c1, tl.row_group, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
+    reduce_tile<G, BLOCK, IPT, EPL>(tile, c0, c1, tl, false, 0, 0, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
     if (!more) break;
     __syncthreads();  // the tile's LDS is free again
     tile = next;
@@ -928,26 +1038,60 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
 #else
   const int tile = tile_of_block(blockIdx.x, tl.xcd_shift);
   if (tile >= num_tiles) return;
-  int2 c0, c1;
-  if (coords != nullptr) {
-    c0 = coords[tile];
-    c1 = coords[tile + 1];
-  } else {
-    __shared__ int2 s_coord[2];
-    {
-      const int w = (int)threadIdx.x / WAVE;
-      if (BLOCK >= 2 * WAVE) {  // the first two wavefronts search one boundary each
-        if (w < 2) {
-          const int2 c = wave_tile_boundary(tile + w, tl, row_end, num_rows, nnz);
-          if ((threadIdx.x & (WAVE - 1)) == 0) s_coord[w] = c;
+  __shared__ int2 s_coord[2];
+  __shared__ int s_split[2];
+  int2 c0 = make_int2(0, 0), c1 = make_int2(0, 0);
+  int split0 = 0, split1 = 0;
+  bool have = false, check = false;
+  if (source != TILES_SEARCHED) {
+    // Read through the scalar cache, as a kernel argument would be: one request per block, no vector
+    // registers.  An entry another block of this launch replaces at the same moment may come back old:
+    // it is then refused like any other stale entry.
+    typedef const __attribute__((address_space(4))) int* TableWords;
+    const TableWords entries = (TableWords)coords + 2 * tile;
+    c0 = make_int2(entries[0], entries[1]);
+    c1 = make_int2(entries[2], entries[3]);
+    have = true;
+    if (source == TILES_CONFIRMED) {
+      split0 = ((TableWords)splits)[tile];
+      split1 = ((TableWords)splits)[tile + 1];
+      // whatever the table held, a tile is only loaded from inside the matrix and never outgrows the block
+      const bool sane = c0.x >= 0 && c0.x <= num_rows && c0.y >= 0 && c0.y <= nnz && c1.x >= c0.x && c1.x <= num_rows &&
+                        c1.y >= c0.y && c1.y <= nnz && (c1.x - c0.x) + (c1.y - c0.y) <= BLOCK * IPT && split0 >= 0 &&
+                        split0 <= num_rows && split1 >= 0 && split1 <= num_rows;
+      have = check = sane;
+    }
+  }
+  // Straight-line: the tile as the table has it; behind it, for a block without usable entries, the search
+  // and the tile code a second time (a loop around one copy keeps every kernel argument and everything
+  // derived from the thread id in registers through the whole tile: 12 scalar spills and up to 17 more
+  // vector registers, 3 % of the kernel on the 3-D stencil).
+  if (have) {
+    const bool refused = reduce_tile<G, BLOCK, IPT, EPL>(tile, c0, c1, tl, check, split0, split1, num_rows, row_end, nnz,
+                                                         p, carry_row, carry_val, agg_partials);
+    if (!refused) return;
+    __syncthreads();  // every thread has read the verdict; the tile's LDS is free again
+  }
+  {
+    const int w = (int)threadIdx.x / WAVE;
+    if (BLOCK >= 2 * WAVE) {  // the first two wavefronts search one boundary each
+      if (w < 2) {
+        int split;
+        const int2 c = wave_tile_boundary(tile + w, tl, row_end, num_rows, nnz, split);
+        if ((threadIdx.x & (WAVE - 1)) == 0) {
+          s_coord[w] = c;
+          s_split[w] = split;
         }
-      } else {
-        const int2 a = wave_tile_boundary(tile, tl, row_end, num_rows, nnz);
-        const int2 b = wave_tile_boundary(tile + 1, tl, row_end, num_rows, nnz);
-        if (threadIdx.x == 0) {
-          s_coord[0] = a;
-          s_coord[1] = b;
-        }
+      }
+    } else {
+      int sa, sb;
+      const int2 a = wave_tile_boundary(tile, tl, row_end, num_rows, nnz, sa);
+      const int2 b = wave_tile_boundary(tile + 1, tl, row_end, num_rows, nnz, sb);
+      if (threadIdx.x == 0) {
+        s_coord[0] = a;
+        s_coord[1] = b;
+        s_split[0] = sa;
+        s_split[1] = sb;
       }
     }
     __syncthreads();
@@ -957,12 +1101,17 @@ reduce_kernel(const int2* __restrict__ coords, const Tiling tl, const int num_ro
     c0.y = __builtin_amdgcn_readfirstlane(c0.y);
     c1.x = __builtin_amdgcn_readfirstlane(c1.x);
     c1.y = __builtin_amdgcn_readfirstlane(c1.y);
-    if (coords_out != nullptr && threadIdx.x == 0) {
-      coords_out[tile] = c0;
-      if (tile == num_tiles - 1) coords_out[num_tiles] = c1;
+    if (threadIdx.x == 0) {
+      coords[tile] = c0;
+      splits[tile] = s_split[0];
+      if (tile == num_tiles - 1) {
+        coords[num_tiles] = c1;
+        splits[num_tiles] = s_split[1];
+      }
     }
+    reduce_tile<G, BLOCK, IPT, EPL>(tile, c0, c1, tl, false, 0, 0, num_rows, row_end, nnz, p, carry_row, carry_val,
+                                    agg_partials);
   }
-  reduce_tile<G, BLOCK, IPT, EPL>(tile, c0, c1, tl.row_group, num_rows, row_end, nnz, p, carry_row, carry_val, agg_partials);
 #endif
 }
 

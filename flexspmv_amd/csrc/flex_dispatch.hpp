@@ -171,7 +171,7 @@ struct Dispatch {
     int carry_blocks;
     bool search_in_blocks;
     bool single_fixup;
-    size_t off_coords, off_carry_row, off_carry_val, off_partials, off_block_partials, off_ticket, total;
+    size_t off_coords, off_splits, off_carry_row, off_carry_val, off_partials, off_block_partials, off_ticket, total;
   };
 
   // Row-snapped tiles pay with smaller tiles (capacity minus the slack a boundary may be moved by), so
@@ -222,6 +222,8 @@ struct Dispatch {
     size_t off = 0;
     l.off_coords = off;
     if (REDUCER) off += align_up(sizeof(int2) * ((size_t)l.num_tiles + 1));
+    l.off_splits = off;
+    if (REDUCER) off += align_up(sizeof(int) * ((size_t)l.num_tiles + 1));
     l.off_carry_row = off;
     if (REDUCER) off += align_up(sizeof(int) * (size_t)l.num_tiles);
     l.off_carry_val = off;
@@ -318,6 +320,7 @@ struct Dispatch {
       const int num_rows = (int)a->num_rows;
       const int* row_end = a->row_end_offsets + 1;  // CSR pointer -> row END offsets
       int2* coords = (int2*)(ws + l.off_coords);
+      int* splits = (int*)(ws + l.off_splits);
       int* carry_row = (int*)(ws + l.off_carry_row);
       V* carry_val = (V*)(ws + l.off_carry_val);
       unsigned* ticket = (unsigned*)(ws + l.off_ticket);
@@ -325,11 +328,36 @@ struct Dispatch {
         fprintf(stderr, "[flexspmv] reducer launch: %d rows, %d non-zeros, %d tiles of %d merge items (capacity %d, snap slack %d), "
                 "%zu bytes of scratch\n", num_rows, nnz, l.num_tiles, l.tiling.nominal, TILE, l.tiling.snap_slack, l.total);
 
-      if (!l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0) {
+      // Where the blocks take their boundaries from.
+      //   From the table the launch before left in this scratch, each block confirming its two entries against
+      //   this launch's row pointer and searching where they do not hold (first launch, another matrix): no
+      //   search kernel, no search in front of the loads.  The default for launches whose blocks would search
+      //   themselves (spring-mass 100^3: step 30.3 -> 28.2 us) and for launches with boundaries on their
+      //   diagonals (R-MAT scale 22: 358.5 -> 348.5 us; the confirmation costs its long-lived blocks 2 us).
+      //   FLEXSPMV_FLAG_CONFIRM_TILES asks for it everywhere.
+      //   From a search kernel in front of the reducer: the default for large launches with row-snapped tiles,
+      //   whose many short-lived blocks pay more for the confirmation (Poisson 256^3: reducer 303.5 -> 309.1
+      //   us) than the 9 us kernel costs beside them, if the reducer's own time is what counts (the step is
+      //   314.8 us confirmed against 316.7).  FLEXSPMV_FLAG_SEARCH_TILES asks for a search on every launch
+      //   everywhere: by the kernel, or inside the blocks of small launches.
+      //   From the table as it is: FLEXSPMV_FLAG_REUSE_TILES, the caller vouches for it.
+      int source;
+      if ((a->flags & FLEXSPMV_FLAG_REUSE_TILES) != 0) source = TILES_FROM_TABLE;
+      else if ((a->flags & FLEXSPMV_FLAG_SEARCH_TILES) != 0) source = l.search_in_blocks ? TILES_SEARCHED : TILES_FROM_TABLE;
+      else if ((a->flags & FLEXSPMV_FLAG_CONFIRM_TILES) != 0 || l.search_in_blocks || l.tiling.snap_slack == 0)
+        source = TILES_CONFIRMED;
+      else source = TILES_FROM_TABLE;
+#ifdef FLEX_TUNE_PERSISTENT  // tuning switch: persistent blocks only read the table
+      source = TILES_FROM_TABLE;
+      const bool search_first = (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0;
+#else
+      const bool search_first = source == TILES_FROM_TABLE && (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0;
+#endif
+      if (search_first) {
         constexpr int per_block = SEARCH_BLOCK / SEARCH_GROUP;
         const int search_blocks = (l.num_tiles + 1 + per_block - 1) / per_block;
         hipLaunchKernelGGL(tile_search_kernel, dim3(search_blocks), dim3(SEARCH_BLOCK), 0, stream, l.tiling, row_end,
-                           num_rows, nnz, coords);
+                           num_rows, nnz, coords, splits);
         report("tile_search_kernel", tile_search_kernel, search_blocks, SEARCH_BLOCK);
       }
 #ifdef FLEX_TUNE_PERSISTENT
@@ -337,22 +365,17 @@ struct Dispatch {
 #else
       const int reduce_grid = grid_for_tiles(l.num_tiles, l.tiling.xcd_shift);
 #endif
-      // Small launches: the reducer blocks search their own boundaries and leave them in the table on the
-      // way (one 8-byte store per block), so that a later launch that may reuse the table skips the search.
-      const bool search_here = l.search_in_blocks && (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0;
-      const int2* table = search_here ? nullptr : coords;
-      int2* table_out = search_here ? coords : nullptr;
       // launches with short regular rows (row-snapped tiles) take several neighbouring edges per load
       constexpr int EPL = edges_per_load<G, IPT>();
       const bool wide_loads = EPL > 1 && l.tiling.snap_slack > 0 && nnz >= EPL;
       auto launch_reducer = [&](auto kernel, const char* name) {
         if (timed) {
-          hipExtLaunchKernelGGL(kernel, dim3(reduce_grid), dim3(BLOCK), 0, stream, g_timer.start, g_timer.stop, 0, table,
-                                l.tiling, num_rows, row_end, nnz, p, carry_row, carry_val, partials, table_out, ticket);
+          hipExtLaunchKernelGGL(kernel, dim3(reduce_grid), dim3(BLOCK), 0, stream, g_timer.start, g_timer.stop, 0, coords,
+                                splits, source, l.tiling, num_rows, row_end, nnz, p, carry_row, carry_val, partials, ticket);
           g_timer.armed = true;
         } else {
-          hipLaunchKernelGGL(kernel, dim3(reduce_grid), dim3(BLOCK), 0, stream, table, l.tiling, num_rows, row_end, nnz, p,
-                             carry_row, carry_val, partials, table_out, ticket);
+          hipLaunchKernelGGL(kernel, dim3(reduce_grid), dim3(BLOCK), 0, stream, coords, splits, source, l.tiling, num_rows,
+                             row_end, nnz, p, carry_row, carry_val, partials, ticket);
         }
         report(name, kernel, reduce_grid, BLOCK);
       };
@@ -410,7 +433,7 @@ inline int check_counts(const flexspmv_launch_args* a, int nv, int ni, int no) {
   if (a->struct_size != sizeof(flexspmv_launch_args))
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "struct_size does not match this library's flexspmv_launch_args");
   if ((a->flags & ~(FLEXSPMV_FLAG_TIME_KERNEL | FLEXSPMV_FLAG_REUSE_TILES | FLEXSPMV_FLAG_KEEP_TILES |
-                    FLEXSPMV_FLAG_DEBUG_SYNC)) != 0)
+                    FLEXSPMV_FLAG_DEBUG_SYNC | FLEXSPMV_FLAG_SEARCH_TILES | FLEXSPMV_FLAG_CONFIRM_TILES)) != 0)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "unknown bits in flags");
   if (a->num_value_inputs != nv || a->num_index_inputs != ni || a->num_outputs != no)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "argument counts do not match flexspmv_signature()");

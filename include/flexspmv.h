@@ -34,24 +34,34 @@
 extern "C" {
 #endif
 
-#define FLEXSPMV_ABI_VERSION 4
+#define FLEXSPMV_ABI_VERSION 5
 
 /* Scratch a library keeps for flexspmv_launch_static (bytes, per library and per GPU it is used on). */
 #define FLEXSPMV_STATIC_SCRATCH_BYTES (4u << 20)
 
 /* flexspmv_launch_args.flags */
 #define FLEXSPMV_FLAG_TIME_KERNEL 1u /* attach HIP events to the dominant kernel's dispatch on args->stream */
-/* Skip the tile search: the caller guarantees that the previous launch of this library with this
- * workspace completed, used the same dtype, num_rows, ne and the same, unmodified row_end_offsets, and
- * that nothing else wrote to the workspace since.  The tile table left in the workspace by that launch
- * is then reused (the reference recomputes it on every call, include/merged_spmv_kernels.cuh:60-99;
- * a solver iterating on a fixed sparsity pattern needs it once). */
+/* The tile table.  A launch of a library with a reducer cuts the merge path into tiles; the boundaries
+ * are what the reference searches for on every call (include/merged_spmv_kernels.cuh:60-99).  Here every
+ * launch leaves them in its workspace, and a later launch on that workspace can try them: each block takes
+ * the two boundaries of its tile from the table, loads the tile, and checks with three row ends per
+ * boundary - fetched together with the tile - that a search on this launch's row_end_offsets would return
+ * exactly them.  Where that holds (a solver loop, a time stepper: the same matrix again) no search runs;
+ * where it does not (first launch on a workspace, another matrix, a workspace that held anything else)
+ * the block searches and nothing of the table is used.  Results never depend on what the workspace held.
+ * This is the default for launches of at most 4096 tiles and for launches whose boundaries stay on their
+ * diagonals (flexspmv_tiling: snap_slack == 0); large launches with row-snapped tiles run a search kernel
+ * in front of the reducer by default (their short-lived blocks pay more for the check than the kernel
+ * costs beside them).  For speed, give every matrix that is launched repeatedly a workspace of its own.
+ *
+ * FLEXSPMV_FLAG_REUSE_TILES: skip the check as well.  The caller guarantees that the previous launch of this
+ * library with this workspace completed, used the same dtype, num_rows, ne and the same, unmodified
+ * row_end_offsets, and that nothing else wrote to the workspace since. */
 #define FLEXSPMV_FLAG_REUSE_TILES 2u
-/* Every launch of a library with a reducer leaves its tile table (int32 pairs (rows, non-zeros) for tile
- * boundaries 0 .. num_tiles) at the start of the workspace: large launches from the search kernel, small
- * ones from the reducer blocks that search their own boundaries.  It can be read back and compared with
- * a CPU merge-path search (see flexspmv_tiling for the diagonals).  This flag is accepted and changes
- * nothing (it used to ask small launches for the table). */
+/* The table is int32 pairs (rows, non-zeros) for tile boundaries 0 .. num_tiles at the start of the
+ * workspace.  It can be read back after a launch and compared with a CPU merge-path search (see
+ * flexspmv_tiling for the diagonals).  This flag is accepted and changes nothing (it used to ask small
+ * launches for the table). */
 #define FLEXSPMV_FLAG_KEEP_TILES 4u
 /* The reference's debug_synchronous argument (cuda_template/reducer/merged_spmv_template.cuh:106-124,131-137):
  * every kernel of the launch is reported on stderr (grid, block, static LDS bytes, registers) and the stream is
@@ -59,6 +69,12 @@ extern "C" {
  * environment variable FLEXSPMV_DEBUG_LAUNCH=1 turns the same on for every launch of the process.  While the
  * stream is being captured the report is printed and the synchronization left out. */
 #define FLEXSPMV_FLAG_DEBUG_SYNC 8u
+/* Do not try the table of an earlier launch: for callers whose row structure changes from launch to launch,
+ * where trying it would fail in every block.  Large launches then run a search kernel in front of the reducer
+ * (one search per boundary instead of two per block), small ones search inside the blocks. */
+#define FLEXSPMV_FLAG_SEARCH_TILES 16u
+/* Try the table of an earlier launch (see above) also where the default is a search kernel. */
+#define FLEXSPMV_FLAG_CONFIRM_TILES 32u
 
 /* Value types a library may have been generated for (flexspmv_launch_args.dtype). */
 enum flexspmv_dtype { FLEXSPMV_F32 = 0, FLEXSPMV_F64 = 1, FLEXSPMV_I64 = 2 };
@@ -86,9 +102,10 @@ enum flexspmv_status {
  *   row_end_offsets  int32[num_rows + 1] with a leading 0 (CSR row pointer); ignored (may be NULL) by
  *                  libraries without a reducer.
  *   ne             number of edges (non-zeros); must be > 0.
- *   workspace      scratch of at least flexspmv_workspace_bytes(...) bytes, 256-byte aligned.  Its contents
- *                  mean nothing to the caller; they only have to be left alone between two launches when
- *                  the second one carries FLEXSPMV_FLAG_REUSE_TILES.
+ *   workspace      scratch of at least flexspmv_workspace_bytes(...) bytes, 256-byte aligned, uninitialised
+ *                  or in whatever state an earlier launch left it.  Its contents mean nothing to the caller;
+ *                  they only have to be left alone between two launches when the second one carries
+ *                  FLEXSPMV_FLAG_REUSE_TILES (and are worth leaving alone otherwise: see the tile table).
  *   stream         hipStream_t to launch on (NULL = default stream).  The call is asynchronous.
  */
 typedef struct flexspmv_launch_args {
@@ -151,8 +168,8 @@ int flexspmv_last_kernel_ms(float* ms);
  *                        boundary is that row start.  snap_slack = 0: boundaries stay on their diagonals.
  *   out[4] tile_capacity merge items a block can hold (threads x items per thread of the policy); at least
  *                        nominal + snap_slack, and more where a cap on the rows per tile shortens nominal
- *   out[5] search_in_blocks  1 when the reducer blocks search their own boundaries instead of a search
- *                        kernel (the tile table is left in the workspace either way), else 0
+ *   out[5] search_in_blocks  1 when a launch with FLEXSPMV_FLAG_SEARCH_TILES searches inside the reducer blocks,
+ *                        0 when it runs a search kernel (launches without the flag never run one)
  * For libraries without a reducer the tiles are plain edge ranges of `nominal` edges.
  * Returns FLEXSPMV_OK, FLEXSPMV_ERR_BAD_DTYPE or FLEXSPMV_ERR_TOO_LARGE. */
 int flexspmv_tiling(int32_t dtype, int64_t num_rows, int64_t ne, int32_t out[6]);

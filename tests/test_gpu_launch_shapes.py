@@ -19,7 +19,7 @@ import pytest
 torch = pytest.importorskip("torch")
 
 from flexspmv_amd import graphs
-from flexspmv_amd.binding import HipExtension
+from flexspmv_amd.binding import FLAG_SEARCH_TILES, HipExtension
 from tests import test_gpu_parity as parity
 from tests import test_gpu_tile_table as tile_table
 from tests.launch_shapes.build_launch_shapes import GRAPHS, VARIANTS, library
@@ -41,6 +41,9 @@ def variant_extension(variant, name):
             raise RuntimeError(f"{path} is not built: run __graft_entry__.build() "
                                "(or tests/launch_shapes/build_launch_shapes.py)")
         _extensions[key] = HipExtension(path, allow_variant=True)
+        # these builds exist for the route with a search kernel and a fix-up block per 256 tiles: every launch
+        # of theirs searches all boundaries afresh (the default would try the table of the launch before)
+        _extensions[key].extra_flags = FLAG_SEARCH_TILES
     return _extensions[key]
 
 
