@@ -191,35 +191,24 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
         step_ms.append(e0.elapsed_time(e1))
     step_ms.sort()
 
-    # Where the blocks of a launch take their tile boundaries from is a policy of the library (flexspmv.h: the tile
-    # table): most launches try the table the launch before left in their scratch and confirm it, block by block,
-    # against the row pointer they are given - the timed region above follows the warm-up on the same matrix, so
-    # its blocks confirm and no search runs -, large launches with row-snapped tiles run a search kernel first.
-    # Beside the default, the same K launches with every boundary searched afresh on every launch, as the
-    # reference does, with the table confirmed ...
-    ms_per_step_search = ms_per_step_confirm = None
-    default_source = None
+    # Launches find the tile table of the launch before in their scratch and confirm it, block by block,
+    # against the row pointer they are given (flexspmv.h: the tile table); the timed region above follows the
+    # warm-up on the same matrix, so its blocks confirm and no search runs.  Beside it: the same K launches
+    # with every boundary searched afresh on every launch, as the reference does (a search kernel in front of
+    # large launches) ...
+    ms_per_step_search = None
     if ext.signature["has_reducer"]:
-        from flexspmv_amd.binding import DTYPE_CODES, FLAG_CONFIRM_TILES, FLAG_SEARCH_TILES
-        import ctypes
-        shape = (ctypes.c_int32 * 6)()
-        ext._lib.flexspmv_tiling(DTYPE_CODES[str(next(iter(w.tensors.values())).dtype)], int(w.num_rows), int(w.ne), shape)
-        default_source = "table confirmed in the blocks" if shape[5] == 1 or shape[2] == 0 else "search kernel"
-
-        def with_flag(flag):
-            ext.extra_flags |= flag
-            warm_up()
-            t0 = time.perf_counter()
-            for _ in range(steps):
-                o = ext.merged_spmv_launch(*args)
-            torch.cuda.synchronize()
-            ms = (time.perf_counter() - t0) * 1e3 / steps
-            ext.extra_flags &= ~flag
-            for x, y in zip(outs, o):
-                assert torch.equal(x, y), "the source of the tile boundaries changed the result"
-            return ms
-        ms_per_step_search = with_flag(FLAG_SEARCH_TILES)
-        ms_per_step_confirm = with_flag(FLAG_CONFIRM_TILES)
+        from flexspmv_amd.binding import FLAG_SEARCH_TILES
+        ext.extra_flags |= FLAG_SEARCH_TILES
+        warm_up()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            outs_search = ext.merged_spmv_launch(*args)
+        torch.cuda.synchronize()
+        ms_per_step_search = (time.perf_counter() - t0) * 1e3 / steps
+        ext.extra_flags &= ~FLAG_SEARCH_TILES
+        for o, r in zip(outs, outs_search):
+            assert torch.equal(o, r), "launch that searched every boundary differs from a launch that confirmed the table"
     # ... and with the table taken on the caller's word, without the confirmation
     ms_per_step_reuse = None
     if ext.signature["has_reducer"]:
@@ -237,17 +226,27 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
     # the dominant kernel alone: HIP events attached to its dispatch inside the library, on the launch stream.
     # Every timed launch is issued between two untimed ones, so that the kernel runs in a busy stream as it
     # does in the K-step region (reading its events back idles the GPU for a moment).
-    warm_up()
-    kernel_ms = []
-    for _ in range(steps):
-        ext.merged_spmv_launch(*args)
-        ext.time_kernel = True
-        ext.merged_spmv_launch(*args)
-        ext.time_kernel = False
-        ext.merged_spmv_launch(*args)
-        kernel_ms.append(ext.last_kernel_ms())
+    def kernel_series():
+        warm_up()
+        series = []
+        for _ in range(steps):
+            ext.merged_spmv_launch(*args)
+            ext.time_kernel = True
+            ext.merged_spmv_launch(*args)
+            ext.time_kernel = False
+            ext.merged_spmv_launch(*args)
+            series.append(ext.last_kernel_ms())
+        return series
+    kernel_ms = kernel_series()
     kernel_ms_mean = sum(kernel_ms) / len(kernel_ms)
     kernel_ms.sort()
+    # the same kernel in launches that search every boundary first (it then only reads the table)
+    kernel_ms_search = None
+    if ext.signature["has_reducer"]:
+        ext.extra_flags |= FLAG_SEARCH_TILES
+        series = kernel_series()
+        ext.extra_flags &= ~FLAG_SEARCH_TILES
+        kernel_ms_search = sum(series) / len(series)
 
     dtype = str(next(iter(w.tensors.values())).dtype)
     machine = None
@@ -276,11 +275,9 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
     if machine:
         result["machine"] = machine
     if ms_per_step_search is not None:
-        result["tile_boundaries_by_default"] = default_source
         result["ms_per_step_search_every_launch"] = ms_per_step_search
         result["gbs_search_every_launch"] = w.algorithmic_bytes / ms_per_step_search / 1e6
-        result["ms_per_step_table_confirmed"] = ms_per_step_confirm
-        result["gbs_table_confirmed"] = w.algorithmic_bytes / ms_per_step_confirm / 1e6
+        result["kernel_ms_search_every_launch"] = kernel_ms_search
     if ms_per_step_reuse is not None:
         result["ms_per_step_tile_reuse"] = ms_per_step_reuse
         result["gbs_tile_reuse"] = w.algorithmic_bytes / ms_per_step_reuse / 1e6
@@ -361,6 +358,10 @@ def roofline_of(r):
            "kernel_ms_min": r["kernel_ms_min"], "launches": None}
     if traffic:
         out["traffic_source"] = traffic["source"]
+    if r.get("kernel_ms_search_every_launch"):
+        # the kernel of a launch that ran a search first does not confirm the table: its own work without that
+        out["kernel_ms_search_every_launch"] = r["kernel_ms_search_every_launch"]
+        out["frac_search_every_launch"] = r["algorithmic_bytes"] / r["kernel_ms_search_every_launch"] / 1e6 / HBM_PEAK_GBS
     if r.get("machine"):
         # the same bytes in the same tiles without the arithmetic: how much of the distance to the peak is the machine's
         out["same_mix_without_arithmetic"] = r["machine"]
@@ -512,8 +513,7 @@ def main() -> int:
         entry = {k: r[k] for k in ("workload", "graph", "dtype", "ne", "num_rows", "algorithmic_bytes", "seed", "policy",
                                    "ms_per_step", "ms_per_step_median_of_regions", "regions", "step_ms_median",
                                    "step_ms_min", "gbs", "edges_per_s", "gflops",
-                                   "tile_boundaries_by_default", "ms_per_step_search_every_launch",
-                                   "gbs_search_every_launch", "ms_per_step_table_confirmed", "gbs_table_confirmed",
+                                   "ms_per_step_search_every_launch", "gbs_search_every_launch",
                                    "ms_per_step_tile_reuse", "gbs_tile_reuse") if k in r}
         entry["pct_of_hbm_peak"] = 100.0 * r["gbs"] / HBM_PEAK_GBS
         entry["roofline"] = roofline_of(r)
@@ -559,18 +559,13 @@ def main() -> int:
         line["config"]["library_variant"] = head["library_variant"]
     if "ms_per_step_search_every_launch" in head:
         line["tile_table"] = {
-            "headline": head["tile_boundaries_by_default"] + " (the library's default for this launch; flexspmv.h, the "
-                        "tile table)",
+            "headline": "every block takes its tile's boundaries from the table the launch before left in the scratch and "
+                        "confirms them against this launch's row pointer (three row ends per boundary, fetched with the "
+                        "tile); the K timed launches follow the warm-up on the same matrix, so no search runs in them",
             "search_every_launch": {"ms_per_step": head["ms_per_step_search_every_launch"],
                                     "value": head["gbs_search_every_launch"], "unit": "GB/s",
                                     "note": "FLEXSPMV_FLAG_SEARCH_TILES: every boundary searched on every launch, as the "
-                                            "reference does"},
-            "table_confirmed": {"ms_per_step": head["ms_per_step_table_confirmed"], "value": head["gbs_table_confirmed"],
-                                "unit": "GB/s",
-                                "note": "FLEXSPMV_FLAG_CONFIRM_TILES: every block takes its boundaries from the table the "
-                                        "launch before left in the scratch and confirms them against this launch's row "
-                                        "pointer (three row ends per boundary, fetched with the tile); the timed launches "
-                                        "follow the warm-up on the same matrix, so no search runs in them"},
+                                            "reference does (a search kernel in front of the reducer)"},
             "taken_on_trust": {"ms_per_step": head["ms_per_step_tile_reuse"], "value": head["gbs_tile_reuse"],
                                "unit": "GB/s", "note": "FLEXSPMV_FLAG_REUSE_TILES: the table used without the confirmation"}}
     if "cpu" in head:

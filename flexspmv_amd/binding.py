@@ -36,7 +36,6 @@ FLAG_REUSE_TILES = 2
 FLAG_KEEP_TILES = 4
 FLAG_DEBUG_SYNC = 8
 FLAG_SEARCH_TILES = 16
-FLAG_CONFIRM_TILES = 32
 DTYPE_CODES = {"float32": 0, "float64": 1, "int64": 2}
 EXPORTED_SYMBOLS = ("flexspmv_launch", "flexspmv_workspace_bytes", "flexspmv_signature",
                     "flexspmv_last_error", "flexspmv_abi_version", "flexspmv_last_kernel_ms", "flexspmv_tiling",

@@ -167,8 +167,12 @@ __device__ __forceinline__ int2 boundary_from_split(int t, const Tiling& tl, int
   const int diag = (int)min(d, (long long)num_rows + nnz);
   const int lo = max(diag - nnz, 0);
   const int hi = min(diag, num_rows);
-  ok = split >= lo && split <= hi && (split == hi || end_at + split + 1 > diag) &&
-       (split == lo || end_before + split <= diag);
+  // every condition as the sign of a difference, so that a block's verdict is a handful of independent
+  // scalar instructions and one OR instead of a chain of compares and branches
+  const int in_bracket = (split - lo) | (hi - split);                                    // >= 0: lo <= split <= hi
+  const int stops_here = split == hi ? 0 : (end_at + split - diag);                     // >= 0: g(split) > diag
+  const int not_before = split == lo ? 0 : (diag - end_before - split);                 // >= 0: g(split - 1) <= diag
+  ok = (in_bracket | stops_here | not_before) >= 0;
   int2 c = make_int2(split, diag - split);
   if (tl.snap_slack > 0 && t > 0 && t < tl.num_tiles) {
     const int xs = split & ~tl.snap_mask;
@@ -499,22 +503,31 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const Tiling& tl, cons
   auto slot_of = [&](const int k) { return (k / EPL) * (EPL * BLOCK) + tid * EPL + (k % EPL); };
 
   // 0: for a tile table that has to be confirmed, the three row ends that decide a boundary (the rows before
-  // and at the split, and the row before the one a snap moves the boundary to): lanes 0-2 of the first
-  // wavefront fetch them for the tile's start, lanes 0-2 of the second for its end (a block of one wavefront:
-  // lanes 0-2 and 3-5).  Issued in front of the tile's loads, they are back first, and the verdict is worked
-  // out while the tile's data are on the way.
+  // and at the split, and the row before the one a snap moves the boundary to).  The first wavefront fetches
+  // them for the tile's start, the second for its end (a block of one wavefront: both), through the scalar
+  // cache - the row pointer does not change during a launch -, so that they are counted apart from the
+  // tile's vector loads: the verdict waits for these three words only and is worked out while the tile's
+  // data are on the way.
   constexpr int CHECKERS = NW >= 2 ? 2 : 1;  // wavefronts that check a boundary
   const int wave_uniform = __builtin_amdgcn_readfirstlane(wave);  // the same number, known to be one per wavefront
   const bool checker = check && wave_uniform < CHECKERS;
-  int check_value = 0;
-  if (checker) {
-    // which of the three rows a lane fetches, without branches: a handful of instructions in front of the
-    // tile's loads (lanes past the ones that count repeat the last row)
-    const bool of_end = CHECKERS == 2 ? wave_uniform == 1 : lane >= 3;
-    const int split = of_end ? split1 : split0;
-    const int part = min(CHECKERS == 2 || lane < 3 ? lane : lane - 3, 2);
-    const int row = (part == 2 ? (split & ~tl.snap_mask) : split) - (part != 1 ? 1 : 0);
-    check_value = row_end[min(max(row, 0), num_rows - 1)];
+  // (Like every load here they are not under a branch - the compiler would wait for them where the branch
+  // ends, in front of the tile's loads: a launch that does not check reads the first row end three times.)
+  int ends_a[3], ends_b[3] = {0, 0, 0};  // of this wavefront's boundary (a block of one wavefront: ends_b the tile's end)
+  {
+    typedef const __attribute__((address_space(4))) int* RowEnds;
+    const RowEnds ends = (RowEnds)row_end;
+    auto fetch = [&](const int split, int (&out)[3]) {
+      out[0] = ends[min(max(split - 1, 0), num_rows - 1)];
+      out[1] = ends[min(max(split, 0), num_rows - 1)];
+      out[2] = ends[min(max((split & ~tl.snap_mask) - 1, 0), num_rows - 1)];
+    };
+    if constexpr (CHECKERS == 2) {
+      fetch(wave_uniform == 0 ? split0 : split1, ends_a);
+    } else {
+      fetch(split0, ends_a);
+      fetch(split1, ends_b);
+    }
   }
 
   // 1: first-level loads.  A tile holds Z <= TILE non-zeros; lanes past Z re-read the tile's last
@@ -611,19 +624,13 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const Tiling& tl, cons
     if constexpr (CHECKERS == 2) {
       bool ok;
       const int2 n = boundary_from_split(tile + wave_uniform, tl, num_rows, nnz, wave_uniform == 0 ? split0 : split1,
-                                         __builtin_amdgcn_readlane(check_value, 0),
-                                         __builtin_amdgcn_readlane(check_value, 1),
-                                         __builtin_amdgcn_readlane(check_value, 2), ok);
+                                         ends_a[0], ends_a[1], ends_a[2], ok);
       const int2 c = wave_uniform == 0 ? c0 : c1;
       confirmed = ok && n.x == c.x && n.y == c.y;
     } else {
       bool ok0, ok1;
-      const int2 n0 = boundary_from_split(tile, tl, num_rows, nnz, split0, __builtin_amdgcn_readlane(check_value, 0),
-                                          __builtin_amdgcn_readlane(check_value, 1),
-                                          __builtin_amdgcn_readlane(check_value, 2), ok0);
-      const int2 n1 = boundary_from_split(tile + 1, tl, num_rows, nnz, split1, __builtin_amdgcn_readlane(check_value, 3),
-                                          __builtin_amdgcn_readlane(check_value, 4),
-                                          __builtin_amdgcn_readlane(check_value, 5), ok1);
+      const int2 n0 = boundary_from_split(tile, tl, num_rows, nnz, split0, ends_a[0], ends_a[1], ends_a[2], ok0);
+      const int2 n1 = boundary_from_split(tile + 1, tl, num_rows, nnz, split1, ends_b[0], ends_b[1], ends_b[2], ok1);
       confirmed = ok0 && ok1 && n0.x == c0.x && n0.y == c0.y && n1.x == c1.x && n1.y == c1.y;
     }
     stale_bit = confirmed ? 0 : 2;
@@ -1056,9 +1063,12 @@ reduce_kernel(int2* coords, int* splits, const int source, const Tiling tl, cons
       split0 = ((TableWords)splits)[tile];
       split1 = ((TableWords)splits)[tile + 1];
       // whatever the table held, a tile is only loaded from inside the matrix and never outgrows the block
-      const bool sane = c0.x >= 0 && c0.x <= num_rows && c0.y >= 0 && c0.y <= nnz && c1.x >= c0.x && c1.x <= num_rows &&
-                        c1.y >= c0.y && c1.y <= nnz && (c1.x - c0.x) + (c1.y - c0.y) <= BLOCK * IPT && split0 >= 0 &&
-                        split0 <= num_rows && split1 >= 0 && split1 <= num_rows;
+      // (signs of differences, OR-ed: no chain of compares in front of the block's first loads; a difference of
+      // two entries only counts where both are in range, and for each entry one of the range terms is exact)
+      const int signs = c0.x | (num_rows - c0.x) | c0.y | (nnz - c0.y) | c1.x | (num_rows - c1.x) | c1.y | (nnz - c1.y) |
+                        split0 | (num_rows - split0) | split1 | (num_rows - split1);
+      const int order = (c1.x - c0.x) | (c1.y - c0.y) | (BLOCK * IPT - (c1.x - c0.x) - (c1.y - c0.y));
+      const bool sane = signs >= 0 && order >= 0;
       have = check = sane;
     }
   }

@@ -328,25 +328,18 @@ struct Dispatch {
         fprintf(stderr, "[flexspmv] reducer launch: %d rows, %d non-zeros, %d tiles of %d merge items (capacity %d, snap slack %d), "
                 "%zu bytes of scratch\n", num_rows, nnz, l.num_tiles, l.tiling.nominal, TILE, l.tiling.snap_slack, l.total);
 
-      // Where the blocks take their boundaries from.
-      //   From the table the launch before left in this scratch, each block confirming its two entries against
-      //   this launch's row pointer and searching where they do not hold (first launch, another matrix): no
-      //   search kernel, no search in front of the loads.  The default for launches whose blocks would search
-      //   themselves (spring-mass 100^3: step 30.3 -> 28.2 us) and for launches with boundaries on their
-      //   diagonals (R-MAT scale 22: 358.5 -> 348.5 us; the confirmation costs its long-lived blocks 2 us).
-      //   FLEXSPMV_FLAG_CONFIRM_TILES asks for it everywhere.
-      //   From a search kernel in front of the reducer: the default for large launches with row-snapped tiles,
-      //   whose many short-lived blocks pay more for the confirmation (Poisson 256^3: reducer 303.5 -> 309.1
-      //   us) than the 9 us kernel costs beside them, if the reducer's own time is what counts (the step is
-      //   314.8 us confirmed against 316.7).  FLEXSPMV_FLAG_SEARCH_TILES asks for a search on every launch
-      //   everywhere: by the kernel, or inside the blocks of small launches.
-      //   From the table as it is: FLEXSPMV_FLAG_REUSE_TILES, the caller vouches for it.
-      int source;
+      // Where the blocks take their boundaries from.  By default from the table the launch before left in
+      // this scratch, each block confirming its two entries against this launch's row pointer and searching
+      // where they do not hold (first launch, another matrix): no search kernel, no search in front of the
+      // loads.  Per step, against a search on every launch: Poisson 256^3 316.6 -> 311.9 us (the reducer pays
+      // 0.8 us for the confirmation, the search kernel cost 9), R-MAT scale 22 356.9 -> 345.7, shallow water
+      // 47.6 -> 46.0, spring-mass 100^3 30.6 -> 28.5 (no search in front of every block's loads).
+      // FLEXSPMV_FLAG_SEARCH_TILES: the row structure changes from launch to launch, so nothing is tried: a
+      // search kernel for large launches, the blocks' own search for small ones (where a kernel for it costs
+      // more than the search).  FLEXSPMV_FLAG_REUSE_TILES: the caller vouches for the table.
+      int source = TILES_CONFIRMED;
       if ((a->flags & FLEXSPMV_FLAG_REUSE_TILES) != 0) source = TILES_FROM_TABLE;
       else if ((a->flags & FLEXSPMV_FLAG_SEARCH_TILES) != 0) source = l.search_in_blocks ? TILES_SEARCHED : TILES_FROM_TABLE;
-      else if ((a->flags & FLEXSPMV_FLAG_CONFIRM_TILES) != 0 || l.search_in_blocks || l.tiling.snap_slack == 0)
-        source = TILES_CONFIRMED;
-      else source = TILES_FROM_TABLE;
 #ifdef FLEX_TUNE_PERSISTENT  // tuning switch: persistent blocks only read the table
       source = TILES_FROM_TABLE;
       const bool search_first = (a->flags & FLEXSPMV_FLAG_REUSE_TILES) == 0;
@@ -433,7 +426,7 @@ inline int check_counts(const flexspmv_launch_args* a, int nv, int ni, int no) {
   if (a->struct_size != sizeof(flexspmv_launch_args))
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "struct_size does not match this library's flexspmv_launch_args");
   if ((a->flags & ~(FLEXSPMV_FLAG_TIME_KERNEL | FLEXSPMV_FLAG_REUSE_TILES | FLEXSPMV_FLAG_KEEP_TILES |
-                    FLEXSPMV_FLAG_DEBUG_SYNC | FLEXSPMV_FLAG_SEARCH_TILES | FLEXSPMV_FLAG_CONFIRM_TILES)) != 0)
+                    FLEXSPMV_FLAG_DEBUG_SYNC | FLEXSPMV_FLAG_SEARCH_TILES)) != 0)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "unknown bits in flags");
   if (a->num_value_inputs != nv || a->num_index_inputs != ni || a->num_outputs != no)
     return fail(FLEXSPMV_ERR_BAD_ARGUMENT, "argument counts do not match flexspmv_signature()");

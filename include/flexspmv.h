@@ -43,16 +43,13 @@ extern "C" {
 #define FLEXSPMV_FLAG_TIME_KERNEL 1u /* attach HIP events to the dominant kernel's dispatch on args->stream */
 /* The tile table.  A launch of a library with a reducer cuts the merge path into tiles; the boundaries
  * are what the reference searches for on every call (include/merged_spmv_kernels.cuh:60-99).  Here every
- * launch leaves them in its workspace, and a later launch on that workspace can try them: each block takes
+ * launch leaves them in its workspace, and a later launch on that workspace tries them: each block takes
  * the two boundaries of its tile from the table, loads the tile, and checks with three row ends per
  * boundary - fetched together with the tile - that a search on this launch's row_end_offsets would return
  * exactly them.  Where that holds (a solver loop, a time stepper: the same matrix again) no search runs;
  * where it does not (first launch on a workspace, another matrix, a workspace that held anything else)
  * the block searches and nothing of the table is used.  Results never depend on what the workspace held.
- * This is the default for launches of at most 4096 tiles and for launches whose boundaries stay on their
- * diagonals (flexspmv_tiling: snap_slack == 0); large launches with row-snapped tiles run a search kernel
- * in front of the reducer by default (their short-lived blocks pay more for the check than the kernel
- * costs beside them).  For speed, give every matrix that is launched repeatedly a workspace of its own.
+ * For speed, give every matrix that is launched repeatedly a workspace of its own.
  *
  * FLEXSPMV_FLAG_REUSE_TILES: skip the check as well.  The caller guarantees that the previous launch of this
  * library with this workspace completed, used the same dtype, num_rows, ne and the same, unmodified
@@ -73,8 +70,6 @@ extern "C" {
  * where trying it would fail in every block.  Large launches then run a search kernel in front of the reducer
  * (one search per boundary instead of two per block), small ones search inside the blocks. */
 #define FLEXSPMV_FLAG_SEARCH_TILES 16u
-/* Try the table of an earlier launch (see above) also where the default is a search kernel. */
-#define FLEXSPMV_FLAG_CONFIRM_TILES 32u
 
 /* Value types a library may have been generated for (flexspmv_launch_args.dtype). */
 enum flexspmv_dtype { FLEXSPMV_F32 = 0, FLEXSPMV_F64 = 1, FLEXSPMV_I64 = 2 };

@@ -18,7 +18,7 @@ torch = pytest.importorskip("torch")
 
 from flexspmv_amd import graphs
 from flexspmv_amd import workloads as W
-from flexspmv_amd.binding import DTYPE_CODES, FLAG_CONFIRM_TILES, FLAG_SEARCH_TILES, load_named
+from flexspmv_amd.binding import DTYPE_CODES, FLAG_SEARCH_TILES, load_named
 from oracle import build_oracle
 from tests.test_gpu_parity import case_rng
 from tests.util_inputs import STRUCTURES, make_inputs, random_row_structure, row_structure
@@ -134,10 +134,9 @@ def test_tile_table_of_the_two_large_workloads(merge_lib):
 
 
 # ---------------------------------------------------------------------------------------------
-# Where the boundaries come from: a block can try the entries an earlier launch left in the scratch and
-# confirm them against the row pointer it was given (the default for most launches; asked for everywhere
-# here); whatever the scratch held, the launch must give the bits of a launch that searches everything, and
-# leave the oracle's table behind.
+# Where the boundaries come from: by default every block tries the entries an earlier launch left in the
+# scratch and confirms them against the row pointer it was given; whatever the scratch held, the launch
+# must give the bits of a launch that searches everything, and leave the oracle's table behind.
 # ---------------------------------------------------------------------------------------------
 def _launch_args(ext, tensors, row_ptr_gpu, num_rows, num_cols):
     args = []
@@ -183,7 +182,7 @@ def test_any_scratch_contents_give_the_result_of_a_full_search(merge_lib, struct
         args = _launch_args(ext, dev, ptr, nr, nc)
         ext.extra_flags = FLAG_SEARCH_TILES                 # the reference's way: every boundary searched
         full = [o.clone() for o in ext.merged_spmv_launch(*args)]
-        ext.extra_flags = FLAG_CONFIRM_TILES
+        ext.extra_flags = 0
         ws, table, splits = _table_and_splits(ext, tl, ptr)
         assert torch.equal(table, want), (variant, "search")
         good_table, good_splits = table.clone(), splits.clone()
@@ -250,7 +249,7 @@ def test_a_matrix_that_changes_under_the_same_scratch(merge_lib):
                 row_ptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
                 ptr.copy_(torch.from_numpy(row_ptr))
             print(f"case changing matrix {variant} step={step} tiles={tl['num_tiles']}", flush=True)
-            ext.extra_flags = FLAG_CONFIRM_TILES
+            ext.extra_flags = 0
             got = ext.merged_spmv_launch(*args)[0].clone()
             _, table, _ = _table_and_splits(ext, tl, ptr)
             assert torch.equal(table, torch.from_numpy(expected_table(merge_lib, row_ptr, tl)).cuda()), (variant, step)
@@ -258,10 +257,9 @@ def test_a_matrix_that_changes_under_the_same_scratch(merge_lib):
             assert torch.equal(ext.merged_spmv_launch(*args)[0], got), (variant, step)
 
 
-def test_default_source_of_the_boundaries_by_launch_class(capfd):
-    """Which kernels a launch runs by default: small launches and launches with boundaries on their diagonals
-    confirm the table (no search kernel), large launches with row-snapped tiles search with a kernel; the flags
-    override both ways."""
+def test_which_kernels_a_launch_runs(capfd):
+    """By default no launch runs a search kernel (its blocks confirm the table of the launch before, or search
+    themselves); with FLEXSPMV_FLAG_SEARCH_TILES large launches run one and small ones search inside their blocks."""
     from flexspmv_amd.binding import FLAG_DEBUG_SYNC
 
     def kernels(w, flags):
@@ -279,9 +277,8 @@ def test_default_source_of_the_boundaries_by_launch_class(capfd):
     small = W.laplacian_2d_spmv(64)
     snapped = W.poisson_3d_spmv_dot(128)           # 16.7 M merge items: more than 4096 tiles, short regular rows
     skewed = W.rmat_spmv(20)                       # more than 4096 tiles, long rows: boundaries stay on their diagonals
-    assert "tile_search_kernel" not in kernels(small, 0)
+    for w in (small, snapped, skewed):
+        assert "tile_search_kernel" not in kernels(w, 0)
     assert "tile_search_kernel" not in kernels(small, FLAG_SEARCH_TILES)       # searched inside the blocks
-    assert "tile_search_kernel" in kernels(snapped, 0)
-    assert "tile_search_kernel" not in kernels(snapped, FLAG_CONFIRM_TILES)
-    assert "tile_search_kernel" not in kernels(skewed, 0)
+    assert "tile_search_kernel" in kernels(snapped, FLAG_SEARCH_TILES)
     assert "tile_search_kernel" in kernels(skewed, FLAG_SEARCH_TILES)

@@ -159,7 +159,7 @@ def test_launch_rejects_bad_arguments_without_touching_the_gpu():
     err = lambda: lib.flexspmv_last_error().decode()
     assert lib.flexspmv_launch(None) == -1
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, struct_size=8))) == -1 and "struct_size" in err()
-    assert lib.flexspmv_launch(ctypes.byref(_args(lib, flags=64))) == -1 and "flags" in err()
+    assert lib.flexspmv_launch(ctypes.byref(_args(lib, flags=32))) == -1 and "flags" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, num_value_inputs=1))) == -1 and "counts" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, dtype=2))) == -2 and "Unsupported dtype" in err()
     assert lib.flexspmv_launch(ctypes.byref(_args(lib, ne=0))) == -1 and "non-empty" in err()
