@@ -128,7 +128,7 @@ def machine_mix_rate(ext, w, dtype_name, write_bytes, launches=30):
             "reads_only_ms": ms_read, "reads_only_gbs": tiles * read_per_tile / ms_read / 1e6}
 
 
-def time_workload(w, steps, warmup, library=None, calibrate=False):
+def time_workload(w, steps, warmup, library=None, calibrate=False, compare_sources=True):
     """GPU leg: returns (result dict, outputs of the last launch as numpy arrays)."""
     import torch
 
@@ -197,8 +197,8 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
     # with every boundary searched afresh on every launch, as the reference does (a search kernel in front of
     # large launches) ...
     ms_per_step_search = None
-    if ext.signature["has_reducer"]:
-        from flexspmv_amd.binding import FLAG_SEARCH_TILES
+    from flexspmv_amd.binding import FLAG_SEARCH_TILES
+    if ext.signature["has_reducer"] and compare_sources:
         ext.extra_flags |= FLAG_SEARCH_TILES
         warm_up()
         t0 = time.perf_counter()
@@ -211,7 +211,7 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
             assert torch.equal(o, r), "launch that searched every boundary differs from a launch that confirmed the table"
     # ... and with the table taken on the caller's word, without the confirmation
     ms_per_step_reuse = None
-    if ext.signature["has_reducer"]:
+    if ext.signature["has_reducer"] and compare_sources:
         ext.reuse_tiles = True
         warm_up()   # the launches one by one above let the clocks drop again
         t0 = time.perf_counter()
@@ -242,7 +242,7 @@ def time_workload(w, steps, warmup, library=None, calibrate=False):
     kernel_ms.sort()
     # the same kernel in launches that search every boundary first (it then only reads the table)
     kernel_ms_search = None
-    if ext.signature["has_reducer"]:
+    if ext.signature["has_reducer"] and compare_sources:
         ext.extra_flags |= FLAG_SEARCH_TILES
         series = kernel_series()
         ext.extra_flags &= ~FLAG_SEARCH_TILES
@@ -456,6 +456,9 @@ def main() -> int:
                          "(default: the other four when the headline is the default Poisson run; 'none' for none)")
     ap.add_argument("--all", action="store_true", help="time all the other four workloads (extra JSON key)")
     ap.add_argument("--cpu-runs", type=int, default=5, help="timed runs of the CPU baseline (0 = skip)")
+    ap.add_argument("--default-launches-only", action="store_true",
+                    help="skip the series that search every boundary on every launch and that take the tile table on "
+                         "trust (a kernel trace then holds the default launches only)")
     ap.add_argument("--no-calibration", action="store_true",
                     help="skip the calibration kernel (the workload's reads and writes without arithmetic)")
     ap.add_argument("--library", default=None,
@@ -483,7 +486,8 @@ def main() -> int:
         w = W.matrix_market_spmv(a.mtx, fused_dot=a.mtx_dot)
     else:
         w = W.WORKLOADS[a.workload](size)
-    head, head_outs = time_workload(w, a.steps, a.warmup, library=a.library, calibrate=not a.no_calibration)
+    head, head_outs = time_workload(w, a.steps, a.warmup, library=a.library, calibrate=not a.no_calibration,
+                                    compare_sources=not a.default_launches_only)
     torch.cuda.empty_cache()
     if a.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").fill_(1.0)
@@ -503,7 +507,8 @@ def main() -> int:
     pending = []
     for name in other_names:
         wo = W.WORKLOADS[name](DEFAULT_SIZE[name])
-        r, o = time_workload(wo, a.steps, a.warmup, calibrate=not a.no_calibration)
+        r, o = time_workload(wo, a.steps, a.warmup, calibrate=not a.no_calibration,
+                             compare_sources=not a.default_launches_only)
         torch.cuda.empty_cache()
         pending.append((name, wo, r, o))
     head = cpu_leg(w, head, head_outs, a.cpu_runs)
