@@ -40,6 +40,7 @@
 namespace flex {
 
 constexpr int NUM_XCD = 8;
+constexpr int NUM_CUS = 256;  // MI355X: 8 XCDs of 32 CUs
 
 // Aggregator partials a reducer block leaves per tile: one (its wavefronts' partials are added in the block,
 // in wavefront order).  One per wavefront - no barrier at the end of the block, four times the words for
@@ -385,6 +386,35 @@ constexpr int edges_per_load() {
   return epl;
 }
 
+// LDS of a reducer block.  Fetched values and index words of the tile's edges, one finished total per row
+// end for the merge path (TILE rows: a tile may consist of row ends only), one dump slot per lane for items
+// that close no row.  Where everything fits a modest budget the totals are a region of their own; otherwise
+// they lie over the fetched values and indices together - the walk has read its items from both by then -
+// so that a block needs no more than the larger of the two.  The spring-mass map (two streamed values and an
+// index per edge, three reduced values per row): 24.6 KB + the dump slots instead of 33.9 KB, 6 resident
+// blocks per CU instead of 4.
+#ifndef FLEX_TUNE_SEPARATE_OUT_BYTES
+#define FLEX_TUNE_SEPARATE_OUT_BYTES (20 * 1024)
+#endif
+template <class G, int BLOCK, int IPT>
+struct TileLds {
+  using V = typename G::Value;
+  static constexpr int TILE = BLOCK * IPT;
+  static constexpr int REDN = G::RED_WIDTH > 0 ? G::RED_WIDTH : 1;
+  static constexpr int FVN = G::FETCH_VALUES > 0 ? G::FETCH_VALUES : 1, FIN = G::FETCH_INDICES > 0 ? G::FETCH_INDICES : 1;
+  static constexpr bool MAP_FIRST = G::ROW_WIDTH == 0;
+  static constexpr int FV_ELEMS = (MAP_FIRST && REDN * TILE > FVN * TILE) ? REDN * TILE : FVN * TILE;  // fetched data / contributions
+  static constexpr size_t FV_BYTES = (size_t)FV_ELEMS * sizeof(V), FI_BYTES = (size_t)FIN * TILE * 4;
+  static constexpr size_t OUT_BYTES = (size_t)REDN * TILE * sizeof(V), DUMP_BYTES = (size_t)REDN * WAVE * sizeof(V);
+  static constexpr bool SEPARATE_OUT = FV_BYTES + FI_BYTES + OUT_BYTES + DUMP_BYTES <= (size_t)FLEX_TUNE_SEPARATE_OUT_BYTES;
+  static constexpr size_t FETCH_BYTES = FV_BYTES + FI_BYTES;
+  static constexpr size_t MAIN_BYTES = SEPARATE_OUT ? FETCH_BYTES + OUT_BYTES : (FETCH_BYTES > OUT_BYTES ? FETCH_BYTES : OUT_BYTES);
+  static constexpr size_t RAW_BYTES = MAIN_BYTES + DUMP_BYTES;
+  // blocks of this kernel a CU holds at a time as far as LDS decides it (160 KB per CU; the small arrays
+  // beside the raw buffer and the allocation granularity are worth another half KB per block)
+  static constexpr int RESIDENT_PER_CU = (int)((160 * 1024) / (RAW_BYTES + 512)) < 8 ? (int)((160 * 1024) / (RAW_BYTES + 512)) : 8;
+};
+
 // ----------------------------------------------------------------------------------------------
 // Reducer kernel.  One block per merge tile of at most BLOCK*IPT merge items (R row ends + Z non-zeros),
 // found by the tile search.  Blocks are small and independent; overlap of one block's memory waits
@@ -455,21 +485,11 @@ reduce_tile(const int tile, const int2 c0, const int2 c1, const Tiling& tl, cons
   static_assert(NWORDS <= WAVE, "one wavefront scans the bitmap words");
 #endif
 
-  // LDS.  s_fv / s_fi hold what was fetched for the tile's edges, s_out one finished total per row end for the
-  // merge path (TILE rows: a tile may consist of row ends only), s_dump one slot per lane for items that
-  // close no row.  Where everything fits a modest budget s_out is a region of its own; otherwise it lies over
-  // s_fv and s_fi together - the walk has read its items from both by then - so that a block needs no more
-  // than the larger of the two.  The spring-mass map (two streamed values and an index per edge, three
-  // reduced values per row): 24.6 KB + the dump slots instead of 33.9 KB, 6 resident blocks per CU instead of 4.
-#ifndef FLEX_TUNE_SEPARATE_OUT_BYTES
-#define FLEX_TUNE_SEPARATE_OUT_BYTES (20 * 1024)
-#endif
-  constexpr int FV_ELEMS = (MAP_FIRST && REDN * TILE > FVN * TILE) ? REDN * TILE : FVN * TILE;  // fetched data / contributions
-  constexpr size_t FV_BYTES = (size_t)FV_ELEMS * sizeof(V), FI_BYTES = (size_t)FIN * TILE * 4;
-  constexpr size_t OUT_BYTES = (size_t)REDN * TILE * sizeof(V), DUMP_BYTES = (size_t)REDN * WAVE * sizeof(V);
-  constexpr bool SEPARATE_OUT = FV_BYTES + FI_BYTES + OUT_BYTES + DUMP_BYTES <= (size_t)FLEX_TUNE_SEPARATE_OUT_BYTES;
-  constexpr size_t FETCH_BYTES = FV_BYTES + FI_BYTES;
-  constexpr size_t MAIN_BYTES = SEPARATE_OUT ? FETCH_BYTES + OUT_BYTES : (FETCH_BYTES > OUT_BYTES ? FETCH_BYTES : OUT_BYTES);
+  // LDS (layout: TileLds)
+  using Lds = TileLds<G, BLOCK, IPT>;
+  constexpr size_t FV_BYTES = Lds::FV_BYTES, FETCH_BYTES = Lds::FETCH_BYTES, MAIN_BYTES = Lds::MAIN_BYTES,
+                   DUMP_BYTES = Lds::DUMP_BYTES;
+  constexpr bool SEPARATE_OUT = Lds::SEPARATE_OUT;
   static_assert(FV_BYTES % 16 == 0 && FETCH_BYTES % 16 == 0 && MAIN_BYTES % 16 == 0, "LDS regions stay 16-byte aligned");
   __shared__ __attribute__((aligned(16))) unsigned char s_raw[MAIN_BYTES + DUMP_BYTES];
   V* const s_fv = reinterpret_cast<V*>(s_raw);

@@ -155,7 +155,7 @@ inline int resident_grid(KernelT kernel, int block_threads, GridCache& cache) {
 #define FLEX_TUNE_INBLOCK_MAX_TILES 4096  // launches of at most this many tiles search inside the reducer blocks
 #endif
 #ifndef FLEX_TUNE_SINGLE_FIXUP_MAX_TILES
-#define FLEX_TUNE_SINGLE_FIXUP_MAX_TILES 4096  // ... and fold carries and aggregators in one block
+#define FLEX_TUNE_SINGLE_FIXUP_MAX_TILES 8192  // launches of at most this many tiles fold carries and aggregators in one block
 #endif
 constexpr int SINGLE_FIXUP_BLOCK = 1024;
 
@@ -203,10 +203,27 @@ struct Dispatch {
 #endif
       }
     }
+    const int64_t items = REDUCER ? num_rows + ne : ne;
+#ifndef FLEX_TUNE_NO_ROUND_BALANCE
+    // A launch of a few rounds of blocks (all CUs filled with as many blocks as fit, then again): its last
+    // round should be a full one.  2.35 rounds take the time of 3, so the tiles shrink until there are 3
+    // rounds of them (spring-mass 100^3: 3 909 tiles of 1 776 items -> 4 606 of 1 507, kernel 24.7 -> 23.2 us);
+    // not where that would cost more than a quarter of the tile, and not for launches of more than four
+    // rounds, whose last round is a small part of the whole (the shallow-water launch, 6.5 rounds made 7:
+    // 44.4 -> 46.2 us, the smaller tiles cost more than the round).
+    if (REDUCER) {
+      constexpr int64_t PER_ROUND = (int64_t)NUM_CUS * TileLds<G, BLOCK, IPT>::RESIDENT_PER_CU;
+      const int64_t tiles = (items + t.nominal - 1) / t.nominal;
+      if (tiles > PER_ROUND && tiles < 4 * PER_ROUND && tiles % PER_ROUND != 0) {
+        const int64_t rounds = (tiles + PER_ROUND - 1) / PER_ROUND;
+        const int64_t nominal = (items + rounds * PER_ROUND - 1) / (rounds * PER_ROUND);
+        if (nominal * 4 >= (int64_t)t.nominal * 3) t.nominal = (int)nominal;
+      }
+    }
+#endif
 #ifdef FLEX_TUNE_NOMINAL  // tuning switch: merge items per tile
     if (FLEX_TUNE_NOMINAL <= TILE - t.snap_slack) t.nominal = FLEX_TUNE_NOMINAL;
 #endif
-    const int64_t items = REDUCER ? num_rows + ne : ne;
     t.num_tiles = (int)((items + t.nominal - 1) / t.nominal);
     return t;
   }

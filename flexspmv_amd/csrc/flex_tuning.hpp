@@ -21,7 +21,7 @@
     defined(FLEX_TUNE_SEPARATE_OUT_BYTES) || defined(FLEX_TUNE_SINGLE_FIXUP_MAX_TILES) || defined(FLEX_TUNE_SNAP_BYTES) || \
     defined(FLEX_TUNE_STAGE_WORDS) || defined(FLEX_TUNE_THREAD_SEARCH) || defined(FLEX_TUNE_UNSAFE_BIG_TILE) ||           \
     defined(FLEX_TUNE_XCD_RUN_SHIFT) || defined(FLEX_TUNE_PARTIAL_PER_WAVE) || defined(FLEX_TUNE_TICKET_SUM) ||       \
-    defined(FLEX_TUNE_GATHER_POLICY)
+    defined(FLEX_TUNE_GATHER_POLICY) || defined(FLEX_TUNE_NO_ROUND_BALANCE)
 #define FLEX_TUNING_ACTIVE 1
 #else
 #define FLEX_TUNING_ACTIVE 0
