@@ -155,7 +155,7 @@ inline int resident_grid(KernelT kernel, int block_threads, GridCache& cache) {
 #define FLEX_TUNE_INBLOCK_MAX_TILES 4096  // launches of at most this many tiles search inside the reducer blocks
 #endif
 #ifndef FLEX_TUNE_SINGLE_FIXUP_MAX_TILES
-#define FLEX_TUNE_SINGLE_FIXUP_MAX_TILES 8192  // launches of at most this many tiles fold carries and aggregators in one block
+#define FLEX_TUNE_SINGLE_FIXUP_MAX_TILES 4096  // launches of at most this many tiles fold carries and aggregators in one block
 #endif
 constexpr int SINGLE_FIXUP_BLOCK = 1024;
 
@@ -235,7 +235,9 @@ struct Dispatch {
     l.num_tiles = l.tiling.num_tiles;
     l.flat_blocks = l.num_tiles < MAX_PERSISTENT_BLOCKS ? l.num_tiles : MAX_PERSISTENT_BLOCKS;
     l.search_in_blocks = REDUCER && l.num_tiles <= FLEX_TUNE_INBLOCK_MAX_TILES;
-    l.single_fixup = REDUCER && l.num_tiles <= FLEX_TUNE_SINGLE_FIXUP_MAX_TILES;
+    // ... twice as many where tiles start on rows: hardly a tile carries then, and the block only walks the records
+    // (spring-mass 100^3, 4 606 tiles: 2.6 us; with a carry per tile 8 192 tiles cost one block 20 us)
+    l.single_fixup = REDUCER && l.num_tiles <= FLEX_TUNE_SINGLE_FIXUP_MAX_TILES * (l.tiling.snap_slack > 0 ? 2 : 1);
     size_t off = 0;
     l.off_coords = off;
     if (REDUCER) off += align_up(sizeof(int2) * ((size_t)l.num_tiles + 1));
