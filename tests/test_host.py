@@ -188,6 +188,23 @@ def test_tiling_query():
     assert flat.flexspmv_tiling(0, 5, 100000, out) == 0 and list(out)[1:4] == [2048, 0, 1]
 
 
+def test_tiles_of_a_launch_of_a_few_rounds_fill_its_last_round():
+    """A launch of one to four rounds of blocks (256 CUs x the blocks a CU holds) gets smaller tiles, by a quarter at
+    most, so that the last round is a full one; launches of less than a round or of more than four keep theirs."""
+    out = (ctypes.c_int32 * 6)()
+    spring = _lib("spring_mass")                      # float32: 25.7 KB of LDS per block, 6 blocks per CU -> 1536 per round
+    assert spring.flexspmv_tiling(0, 1_000_000, 5_940_000, out) == 0
+    num_tiles, nominal, slack, _, capacity, _ = list(out)
+    assert nominal + slack < capacity                 # smaller than the largest tile that would fit ...
+    assert 4 * nominal >= 3 * (capacity - slack)      # ... by a quarter at most
+    assert num_tiles == -(-(6_940_000) // nominal) and 3 * 1536 - 8 <= num_tiles <= 3 * 1536
+    assert spring.flexspmv_tiling(0, 10_000, 59_400, out) == 0 and out[1] == 1776     # less than a round: 256 average rows
+    swe = _lib("swe_rusanov")                         # 6.5 rounds: left alone
+    assert swe.flexspmv_tiling(1, 1_999_960, 5_999_842, out) == 0 and (out[0], out[1]) == (8334, 960)
+    poisson = _lib("spmv_dot")                        # 45 rounds
+    assert poisson.flexspmv_tiling(1, 16777216, 117047296, out) == 0 and (out[0], out[1]) == (69701, 1920)
+
+
 def test_workspace_query():
     lib = _lib("spmv_dot")
     small = lib.flexspmv_workspace_bytes(1, 1000, 7000)
