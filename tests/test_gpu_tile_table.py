@@ -282,3 +282,47 @@ def test_which_kernels_a_launch_runs(capfd):
     assert "tile_search_kernel" not in kernels(small, FLAG_SEARCH_TILES)       # searched inside the blocks
     assert "tile_search_kernel" in kernels(snapped, FLAG_SEARCH_TILES)
     assert "tile_search_kernel" in kernels(skewed, FLAG_SEARCH_TILES)
+
+
+def test_captured_launch_replayed_on_a_changing_matrix(merge_lib):
+    """A launch captured into a HIP graph and replayed while the matrix behind its row pointer changes between the
+    replays (same sizes, eager launches and synchronisation in between): every replay confirms what still holds of
+    the table in the captured scratch, searches the rest, and equals an eager launch that searches everything."""
+    rng = np.random.default_rng(91)
+    ir = graphs.get("spmv_dot")
+    nr = 30_000
+    lengths = rng.integers(0, 10, nr)
+    row_ptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    tensors, row_ptr, _, nc, ne = make_inputs(ir, np.dtype("float64"), rng, row_ptr=row_ptr)
+    dev = {k: torch.from_numpy(np.ascontiguousarray(v)).cuda() for k, v in tensors.items()}
+    ptr = torch.from_numpy(row_ptr).cuda()
+    from flexspmv_amd.binding import HipExtension
+    ext = HipExtension(load_named("spmv_dot", build_if_missing=False).lib_path)
+    fresh = HipExtension(ext.lib_path)
+    fresh.extra_flags = FLAG_SEARCH_TILES
+    args = _launch_args(ext, dev, ptr, nr, nc)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ext.merged_spmv_launch(*args)                       # allocates the scratch of that stream
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        y, dot = ext.merged_spmv_launch(*args)
+    for step in range(5):
+        if step > 0:
+            lo = int(rng.integers(0, nr - 3000))
+            part = lengths[lo: lo + 3000].copy()
+            rng.shuffle(part)
+            lengths[lo: lo + 3000] = part
+            row_ptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+            ptr.copy_(torch.from_numpy(row_ptr))
+            if "selector_row_idx" in dev:                   # the row-aligned selector follows the rows
+                dev["selector_row_idx"].copy_(torch.from_numpy(
+                    np.repeat(np.arange(nr, dtype=np.int32), np.diff(row_ptr))))
+        print(f"case captured launch, changing matrix step={step}", flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        want_y, want_dot = fresh.merged_spmv_launch(*args)
+        assert torch.equal(y, want_y) and torch.equal(dot, want_dot), step
