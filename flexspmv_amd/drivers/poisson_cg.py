@@ -16,7 +16,6 @@ def fused_operator(n: int, device="cuda", dtype=torch.float64) -> Tuple[Callable
     """``apply(p) -> (A p, p . A p)`` for the 7-point Laplacian on an n^3 grid, and the vector length."""
     w = W.poisson_3d_spmv_dot(n, dtype=str(dtype).replace("torch.", ""))
     ext = load_named(w.graph, build_if_missing=False)
-    ext.reuse_tiles = True
     names = ext.param_names()
     args = W.launch_arguments(w, names, device)
     xi = names.index("x")
