@@ -441,6 +441,34 @@ def time_edge_list_preparation(w, steps):
     return out
 
 
+def machine_rates(gib: int = 2, reps: int = 20):
+    """TB/s of three library kernels on tensors of `gib` GiB (events around `reps` back-to-back calls)."""
+    import torch
+    n = gib << 27   # float64 elements
+    src = torch.empty(n, dtype=torch.float64, device="cuda:0").fill_(1.0)
+    dst = torch.empty_like(src)
+
+    def rate(call, nbytes):
+        call()
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(reps):
+            call()
+        t1.record()
+        torch.cuda.synchronize()
+        return round(nbytes / (t0.elapsed_time(t1) / reps * 1e-3) / 1e12, 3)
+
+    one = n * 8
+    out = {"tensor_bytes": one, "unit": "TB/s",
+           "write_only_fill": rate(lambda: dst.fill_(1.0), one),
+           "read_only_sum": rate(lambda: src.sum(), one),
+           "read_write_1_to_1_add": rate(lambda: torch.add(src, 1.0, out=dst), 2 * one)}
+    del src, dst
+    torch.cuda.empty_cache()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -467,6 +495,9 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain elementwise copies (dst = src + 1) of 1 GiB, a kernel of known "
                          "traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--machine-rates", action="store_true",
+                    help="also time torch's fill, sum and dst = src + 1 on 2 GiB tensors: what this GPU gives a "
+                         "library's write-only, read-only and 1 : 1 streaming kernels (extra JSON key)")
     ap.add_argument("--formats", action="store_true",
                     help="also time the edge-list preparation kernels on this workload's edge list (extra JSON key)")
     a = ap.parse_args()
@@ -497,6 +528,7 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
+    rates = machine_rates() if a.machine_rates else None
     if a.all:
         other_names = [n for n in ("rmat", "spring_mass", "shallow_water", "laplacian2d") if n != a.workload]
     elif a.others is not None:
@@ -577,6 +609,8 @@ def main() -> int:
         line["cpu_baseline"] = cpu_baseline_of(head)
     if others:
         line["other_workloads"] = others
+    if rates is not None:
+        line["machine_rates"] = rates
     if a.formats:
         line["edge_list_preparation"] = time_edge_list_preparation(w, a.steps)
     if not parity_ok:
