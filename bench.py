@@ -44,6 +44,8 @@ WORKLOAD_NOTES = {
                    "length every force and the energy would be exactly zero",
     "shallow_water": "cells renumbered along a Morton curve through their centroids before the half-edges are "
                      "sorted by destination cell (the triangulation's own numbering has no locality)",
+    "laplacian2d": "the reference's CPU-sized case: 3.4 MB of algorithmic bytes are 0.4 us at the HBM peak, so the step is "
+                   "the latency of its two kernel launches and the roofline fraction says nothing about the kernel",
 }
 
 
