@@ -443,6 +443,50 @@ def time_edge_list_preparation(w, steps):
     return out
 
 
+def torch_sparse_comparison(w, reps: int = 10):
+    """The same product by torch's own kernels, for SpMV workloads: `index_select` of x by the column index (the
+    gather alone) and the sparse-CSR product the installed torch dispatches to its vendor library.  Microseconds
+    per call, events around `reps` back-to-back calls."""
+    import torch
+    from flexspmv_amd import workloads as W
+    from flexspmv_amd.binding import load_named
+    names = load_named(w.graph, build_if_missing=False).param_names()
+    col_name = next((n for n in ("selector_idx", "selector_col_idx") if n in names), None)
+    if col_name is None or "vals" not in names or "x" not in names:
+        return None
+    args = W.launch_arguments(w, names, "cuda:0")
+    x, cols, vals = (args[names.index(n)] for n in ("x", col_name, "vals"))
+    row_ptr = args[names.index("row_end_offsets")]
+
+    def us(call):
+        call()
+        torch.cuda.synchronize()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(reps):
+            call()
+        t1.record()
+        torch.cuda.synchronize()
+        return round(t0.elapsed_time(t1) / reps * 1e3, 1)
+
+    gathered = torch.empty(cols.numel(), dtype=x.dtype, device=x.device)
+    out = {"unit": "us per call",
+           "index_select_of_x_by_column": us(lambda: torch.index_select(x, 0, cols, out=gathered))}
+    del gathered
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        matrix = torch.sparse_csr_tensor(row_ptr, cols, vals, size=(w.num_rows, w.num_cols))
+    column = x.unsqueeze(1)
+    if w.graph == "spmv_dot":
+        out["sparse_csr_product_and_dot"] = us(lambda: torch.dot(x, (matrix @ column).squeeze(1)))
+    else:
+        out["sparse_csr_product"] = us(lambda: matrix @ column)
+    del matrix
+    torch.cuda.empty_cache()
+    return out
+
+
 def machine_rates(gib: int = 2, reps: int = 20):
     """TB/s of three library kernels on tensors of `gib` GiB (events around `reps` back-to-back calls)."""
     import torch
@@ -467,6 +511,18 @@ def machine_rates(gib: int = 2, reps: int = 20):
            "read_only_sum": rate(lambda: src.sum(), one),
            "read_write_1_to_1_add": rate(lambda: torch.add(src, 1.0, out=dst), 2 * one)}
     del src, dst
+    # uniformly random 4-byte gathers (index_select, 2^26 int32 indices) from tables of several sizes
+    count = 1 << 26
+    gen = torch.Generator(device="cuda:0").manual_seed(3)
+    gathered = torch.empty(count, dtype=torch.float32, device="cuda:0")
+    out["random_gathers"] = {"unit": "T gathers/s", "indices": count}
+    for table_bytes in (1 << 16, 1 << 22, 1 << 24, 1 << 26):
+        table = torch.rand(table_bytes // 4, device="cuda:0")
+        idx = torch.randint(0, table.numel(), (count,), device="cuda:0", dtype=torch.int32, generator=gen)
+        out["random_gathers"][f"table_of_{table_bytes}_bytes"] = rate(
+            lambda: torch.index_select(table, 0, idx, out=gathered), count)
+        del table, idx
+    del gathered
     torch.cuda.empty_cache()
     return out
 
@@ -497,9 +553,12 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain elementwise copies (dst = src + 1) of 1 GiB, a kernel of known "
                          "traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--torch-sparse", action="store_true",
+                    help="also time torch's own kernels on the headline workload, if it is an SpMV: index_select of x "
+                         "by the column index and the sparse-CSR product (extra JSON key)")
     ap.add_argument("--machine-rates", action="store_true",
-                    help="also time torch's fill, sum and dst = src + 1 on 2 GiB tensors: what this GPU gives a "
-                         "library's write-only, read-only and 1 : 1 streaming kernels (extra JSON key)")
+                    help="also time torch's fill, sum and dst = src + 1 on 2 GiB tensors and its index_select with random "
+                         "indices: what this GPU gives a library's streaming and gathering kernels (extra JSON key)")
     ap.add_argument("--formats", action="store_true",
                     help="also time the edge-list preparation kernels on this workload's edge list (extra JSON key)")
     a = ap.parse_args()
@@ -531,6 +590,7 @@ def main() -> int:
         del src, dst
         torch.cuda.empty_cache()
     rates = machine_rates() if a.machine_rates else None
+    torch_sparse = torch_sparse_comparison(w) if a.torch_sparse else None
     if a.all:
         other_names = [n for n in ("rmat", "spring_mass", "shallow_water", "laplacian2d") if n != a.workload]
     elif a.others is not None:
@@ -613,6 +673,8 @@ def main() -> int:
         line["other_workloads"] = others
     if rates is not None:
         line["machine_rates"] = rates
+    if torch_sparse is not None:
+        line["torch_sparse"] = torch_sparse
     if a.formats:
         line["edge_list_preparation"] = time_edge_list_preparation(w, a.steps)
     if not parity_ok:
